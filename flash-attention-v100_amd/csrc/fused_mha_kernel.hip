@@ -1,0 +1,665 @@
+// FlashAttention-2 forward and backward for gfx950 (CDNA4, wave64, MFMA).
+//
+// Takes the place of the reference's kernel/fused_mha_kernel.cu (forward
+// :20-323, backward :325-735, launchers :891-916) with a different design:
+//
+//   * Every GEMM runs on v_mfma_f32_32x32x16_f16 with fp32 accumulation.
+//   * A wave owns 32 "resident" sequence positions (queries in the forward and
+//     in the dQ pass, keys in the dK/dV pass).  Their rows stay in registers as
+//     MFMA B operands for the whole kernel.  The other sequence dimension is
+//     streamed through LDS in 64-row tiles shared by the 4 waves of a block.
+//   * The first GEMM is computed transposed, tile^T[streamed][resident], so a
+//     lane holds 16 streamed positions of ONE resident position per 32x32
+//     block.  Row statistics (max, sum, logsumexp, delta) are therefore plain
+//     per-lane scalars plus one exchange between the two 32-lane halves.
+//   * The accumulator registers of the first GEMM, rounded to fp16, are
+//     already laid out as the B operand of the second GEMM, so P and dS never
+//     travel through LDS.  The matching A operand (V^T, K^T, Q^T, dO^T) is read
+//     from the same row-major LDS tile with ds_read_b64_tr_b16.
+//   * The backward is split into a dQ pass (query-block parallel) and a dK/dV
+//     pass (key-block parallel): no atomics, no fp32 dQ scratch, deterministic.
+//
+// Layouts: q/k/v/o/do/dq/dk/dv are (B, N, H, D) fp16, lse/delta are (B, H, N)
+// fp32 (reference: kernel/fused_mha_kernel.cu:57-67).
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <math.h>
+
+#include "fused_mha.h"
+
+namespace {
+
+typedef _Float16 half_t;
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef short s4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef float f2v __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;      // 4 waves
+constexpr int kWaves = 4;
+constexpr int kResident = 32;      // resident positions per wave
+constexpr int kBlockRes = kWaves * kResident;  // 128 resident positions per block
+constexpr int kTile = 64;          // streamed rows per LDS tile
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <int D>
+struct TileGeom {
+  static constexpr int kRowBytes = D * 2 + 16;             // padded LDS row
+  static constexpr int kTileBytes = kTile * kRowBytes;
+  static constexpr int kChunksPerRow = D / 8;              // 16-byte chunks
+  static constexpr int kChunksPerThread = kTile * kChunksPerRow / kThreads;
+  static constexpr int kKSteps = D / 16;                   // MFMA k-steps over D
+  static constexpr int kDBlocks = D / 32;                  // 32-row blocks over D
+};
+
+__device__ __forceinline__ f16v mfma(h8 a, h8 b, f16v c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Combine a value with the one held by the lane 32 positions away.
+__device__ __forceinline__ float other_half(float x) {
+  int xi = __float_as_int(x);
+  auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+  // r[0]: lanes 0-31 keep own, lanes 32-63 get lane-32's; r[1] the converse.
+  int mine_or_other = (threadIdx.x & 32) ? r[0] : r[1];
+  return __int_as_float(mine_or_other);
+}
+
+// Global -> registers for one 64-row tile (rows clamped to n-1).
+template <int D>
+__device__ __forceinline__ void tile_load(const half_t* __restrict__ base, long row_stride,
+                                          int row0, int n, h8 (&regs)[TileGeom<D>::kChunksPerThread]) {
+  using G = TileGeom<D>;
+#pragma unroll
+  for (int i = 0; i < G::kChunksPerThread; ++i) {
+    int ch = threadIdx.x + kThreads * i;
+    int r = ch / G::kChunksPerRow;
+    int c = ch % G::kChunksPerRow;
+    int row = min(row0 + r, n - 1);
+    regs[i] = *reinterpret_cast<const h8*>(base + (long)row * row_stride + c * 8);
+  }
+}
+
+// Registers -> LDS (row-major, padded rows).
+template <int D>
+__device__ __forceinline__ void tile_store(char* lds, const h8 (&regs)[TileGeom<D>::kChunksPerThread]) {
+  using G = TileGeom<D>;
+#pragma unroll
+  for (int i = 0; i < G::kChunksPerThread; ++i) {
+    int ch = threadIdx.x + kThreads * i;
+    int r = ch / G::kChunksPerRow;
+    int c = ch % G::kChunksPerRow;
+    *reinterpret_cast<h8*>(lds + r * G::kRowBytes + c * 16) = regs[i];
+  }
+}
+
+// A operand of the first GEMM: rows = 32 streamed positions (row-block rb),
+// k = 16 feature columns of k-step kk.  Lane (i, hh) reads 8 contiguous halves.
+template <int D>
+__device__ __forceinline__ h8 read_rows(const char* lds, int rb, int kk, int lane_row_off) {
+  return *reinterpret_cast<const h8*>(lds + lane_row_off + rb * 32 * TileGeom<D>::kRowBytes + kk * 32);
+}
+
+// A operand of the second GEMM: rows = 32 feature columns (block db), k = 16
+// streamed positions of chunk c16, read transposed out of the row-major tile.
+// The k order matches the accumulator layout of the first GEMM:
+// k index 8*hh + j  <->  streamed row 16*c16 + 8*(j/4) + 4*hh + j%4.
+template <int D>
+__device__ __forceinline__ h8 read_cols(const char* lds, int c16, int db, int lane_tr_off) {
+  using G = TileGeom<D>;
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const char* p = lds + lane_tr_off + c16 * 16 * G::kRowBytes + db * 64;
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p));
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + 8 * G::kRowBytes));
+  return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+__device__ __forceinline__ h8 pack8(const f16v& x, int base) {
+  h8 r;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = (half_t)x[base + j];
+  return r;
+}
+
+// Streamed-row index of accumulator register r in row-block rb for half hh.
+__device__ __forceinline__ int acc_row(int rb, int r, int hh) {
+  return rb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
+}
+
+// Store a [D][32 resident] fp32 accumulator, scaled, as fp16 rows of a
+// (B, N, H, D) tensor.  Lane (i, hh) owns resident row `row`; per 32-feature
+// block it holds features 8*g + 4*hh + 0..3 for g = 0..3.
+template <int D>
+__device__ __forceinline__ void store_resident(half_t* __restrict__ base, long row_stride, int row, int n,
+                                               const f16v (&acc)[TileGeom<D>::kDBlocks], float mul, int hh) {
+  if (row >= n) return;
+  half_t* p = base + (long)row * row_stride;
+#pragma unroll
+  for (int db = 0; db < TileGeom<D>::kDBlocks; ++db) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      h4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (half_t)(acc[db][4 * g + e] * mul);
+      *reinterpret_cast<h4*>(p + db * 32 + 8 * g + 4 * hh) = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Forward.  Block = 128 queries, wave = 32 queries, streams K/V tiles of 64.
+// ---------------------------------------------------------------------------
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(kThreads, 2)
+fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
+                half_t* __restrict__ O, float* __restrict__ LSE, int H, int N, float c, int negate_q) {
+  using G = TileGeom<D>;
+  __shared__ __attribute__((aligned(16))) char smem[4 * G::kTileBytes];  // K0 V0 K1 V1
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = lane & 31, hh = lane >> 5;
+  const int mblk = CAUSAL ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;  // heavy blocks first
+  const int b = blockIdx.y / H, h = blockIdx.y % H;
+  const long rs = (long)H * D;
+  const long head_off = ((long)b * N * H + h) * D;
+  const half_t* Qb = Q + head_off;
+  const half_t* Kb = K + head_off;
+  const half_t* Vb = V + head_off;
+
+  const int m0 = mblk * kBlockRes;
+  const int q0w = m0 + wave * kResident;
+  const int qi = q0w + i;
+
+  h8 qf[G::kKSteps];
+  {
+    const half_t* qp = Qb + (long)min(qi, N - 1) * rs + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+      qf[kk] = *reinterpret_cast<const h8*>(qp + kk * 16);
+      if (negate_q) qf[kk] = -qf[kk];
+    }
+  }
+
+  int nt = (N + kTile - 1) / kTile;
+  if (CAUSAL) nt = min(nt, (min(m0 + kBlockRes, N) - 1) / kTile + 1);
+
+  const int lane_row_off = i * G::kRowBytes + hh * 16;
+  const int lane_tr_off = (4 * hh + ((lane & 15) >> 2)) * G::kRowBytes + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  f16v o[G::kDBlocks];
+#pragma unroll
+  for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  h8 kreg[G::kChunksPerThread], vreg[G::kChunksPerThread];
+  tile_load<D>(Kb, rs, 0, N, kreg);
+  tile_load<D>(Vb, rs, 0, N, vreg);
+  tile_store<D>(smem, kreg);
+  tile_store<D>(smem + G::kTileBytes, vreg);
+  __syncthreads();
+
+  for (int kt = 0; kt < nt; ++kt) {
+    const char* Kl = smem + (kt & 1) * 2 * G::kTileBytes;
+    const char* Vl = Kl + G::kTileBytes;
+    const bool more = kt + 1 < nt;
+    if (more) {
+      tile_load<D>(Kb, rs, (kt + 1) * kTile, N, kreg);
+      tile_load<D>(Vb, rs, (kt + 1) * kTile, N, vreg);
+    }
+    const int key0 = kt * kTile;
+    const bool active = !CAUSAL || key0 <= q0w + kResident - 1;
+    if (active) {
+      f16v s[2];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[rb][r] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < G::kKSteps; ++kk) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(read_rows<D>(Kl, rb, kk, lane_row_off), qf[kk], s[rb]);
+      }
+      const bool need_mask = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
+      if (need_mask) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            int key = key0 + acc_row(rb, r, hh);
+            if ((CAUSAL && key > qi) || key >= N) s[rb][r] = -INFINITY;
+          }
+      }
+      float mx = s[0][0];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[rb][r]);
+      mx = fmaxf(mx, other_half(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = fast_exp2((m_run - m_new) * c);
+      const float mc = m_new * c;
+      m_run = m_new;
+      float rowsum = 0.f;
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float p = fast_exp2(fmaf(s[rb][r], c, -mc));
+          s[rb][r] = p;
+          rowsum += p;
+        }
+      l_run = l_run * alpha + rowsum;
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+      h8 pf[4];
+#pragma unroll
+      for (int c16 = 0; c16 < 4; ++c16) pf[c16] = pack8(s[c16 >> 1], (c16 & 1) * 8);
+#pragma unroll
+      for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+        for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(read_cols<D>(Vl, c16, db, lane_tr_off), pf[c16], o[db]);
+      }
+    }
+    if (more) {
+      char* Kn = smem + ((kt + 1) & 1) * 2 * G::kTileBytes;
+      tile_store<D>(Kn, kreg);
+      tile_store<D>(Kn + G::kTileBytes, vreg);
+    }
+    __syncthreads();
+  }
+
+  const float l_tot = l_run + other_half(l_run);
+  const float inv = 1.f / l_tot;
+  store_resident<D>(O + head_off, rs, qi, N, o, inv, hh);
+  if (hh == 0 && qi < N) LSE[((long)b * H + h) * N + qi] = (m_run * c + __builtin_amdgcn_logf(l_tot)) * kLn2;
+}
+
+// ---------------------------------------------------------------------------
+// delta[b][h][n] = sum_d dO * O in fp32.  One 16-byte chunk per thread.
+// Takes the place of the two PyTorch ops at reference
+// flash_attn_interface.py:43-44 (which work in fp16).
+// ---------------------------------------------------------------------------
+template <int D>
+__global__ void __launch_bounds__(256)
+fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ dO, float* __restrict__ delta,
+                      int H, int N, long rows) {
+  constexpr int kLanesPerRow = D / 8;
+  const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const long row = t / kLanesPerRow;  // (b*N + n)*H + h
+  const int c = (int)(t % kLanesPerRow);
+  float acc = 0.f;
+  if (row < rows) {
+    h8 a = *reinterpret_cast<const h8*>(O + row * D + c * 8);
+    h8 g = *reinterpret_cast<const h8*>(dO + row * D + c * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc = fmaf((float)a[j], (float)g[j], acc);
+  }
+#pragma unroll
+  for (int off = kLanesPerRow / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if (row < rows && c == 0) {
+    const long bn = row / H;
+    const int h = (int)(row % H);
+    const long b = bn / N;
+    const int n = (int)(bn % N);
+    delta[(b * H + h) * N + n] = acc;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward, dQ pass.  Block = 128 queries, wave = 32 queries, streams K/V.
+//   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T o (dP^T - delta), dQ^T += K^T dS^T
+// (formulas: reference kernel/fused_mha_kernel.cu:598-603, 653-656, 680-683).
+// ---------------------------------------------------------------------------
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(kThreads, 2)
+fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
+                   const half_t* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ delta,
+                   half_t* __restrict__ dQ, int H, int N, float c, float scale) {
+  using G = TileGeom<D>;
+  __shared__ __attribute__((aligned(16))) char smem[4 * G::kTileBytes];  // K0 V0 K1 V1
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = lane & 31, hh = lane >> 5;
+  const int mblk = CAUSAL ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
+  const int b = blockIdx.y / H, h = blockIdx.y % H;
+  const long rs = (long)H * D;
+  const long head_off = ((long)b * N * H + h) * D;
+  const half_t* Kb = K + head_off;
+  const half_t* Vb = V + head_off;
+
+  const int m0 = mblk * kBlockRes;
+  const int q0w = m0 + wave * kResident;
+  const int qi = q0w + i;
+  const int qrow = min(qi, N - 1);
+
+  h8 qf[G::kKSteps], dof[G::kKSteps];
+  {
+    const half_t* qp = Q + head_off + (long)qrow * rs + hh * 8;
+    const half_t* gp = dO + head_off + (long)qrow * rs + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+      qf[kk] = *reinterpret_cast<const h8*>(qp + kk * 16);
+      dof[kk] = *reinterpret_cast<const h8*>(gp + kk * 16);
+    }
+  }
+  const float l2 = LSE[((long)b * H + h) * N + qrow] * kLog2e;
+  const float dl = delta[((long)b * H + h) * N + qrow];
+
+  int nt = (N + kTile - 1) / kTile;
+  if (CAUSAL) nt = min(nt, (min(m0 + kBlockRes, N) - 1) / kTile + 1);
+
+  const int lane_row_off = i * G::kRowBytes + hh * 16;
+  const int lane_tr_off = (4 * hh + ((lane & 15) >> 2)) * G::kRowBytes + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  f16v dq[G::kDBlocks];
+#pragma unroll
+  for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
+
+  h8 kreg[G::kChunksPerThread], vreg[G::kChunksPerThread];
+  tile_load<D>(Kb, rs, 0, N, kreg);
+  tile_load<D>(Vb, rs, 0, N, vreg);
+  tile_store<D>(smem, kreg);
+  tile_store<D>(smem + G::kTileBytes, vreg);
+  __syncthreads();
+
+  for (int kt = 0; kt < nt; ++kt) {
+    const char* Kl = smem + (kt & 1) * 2 * G::kTileBytes;
+    const char* Vl = Kl + G::kTileBytes;
+    const bool more = kt + 1 < nt;
+    if (more) {
+      tile_load<D>(Kb, rs, (kt + 1) * kTile, N, kreg);
+      tile_load<D>(Vb, rs, (kt + 1) * kTile, N, vreg);
+    }
+    const int key0 = kt * kTile;
+    const bool active = !CAUSAL || key0 <= q0w + kResident - 1;
+    if (active) {
+      const bool need_mask = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
+      h8 dsf[4];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        f16v s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int kk = 0; kk < G::kKSteps; ++kk) {
+          s = mfma(read_rows<D>(Kl, rb, kk, lane_row_off), qf[kk], s);
+          dp = mfma(read_rows<D>(Vl, rb, kk, lane_row_off), dof[kk], dp);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float p = fast_exp2(fmaf(s[r], c, -l2));
+          if (need_mask) {
+            int key = key0 + acc_row(rb, r, hh);
+            if ((CAUSAL && key > qi) || key >= N) p = 0.f;
+          }
+          s[r] = p * (dp[r] - dl);
+        }
+        dsf[rb * 2] = pack8(s, 0);
+        dsf[rb * 2 + 1] = pack8(s, 8);
+      }
+#pragma unroll
+      for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+        for (int db = 0; db < G::kDBlocks; ++db) dq[db] = mfma(read_cols<D>(Kl, c16, db, lane_tr_off), dsf[c16], dq[db]);
+      }
+    }
+    if (more) {
+      char* Kn = smem + ((kt + 1) & 1) * 2 * G::kTileBytes;
+      tile_store<D>(Kn, kreg);
+      tile_store<D>(Kn + G::kTileBytes, vreg);
+    }
+    __syncthreads();
+  }
+  store_resident<D>(dQ + head_off, rs, qi, N, dq, scale, hh);
+}
+
+// ---------------------------------------------------------------------------
+// Backward, dK/dV pass.  Block = 128 keys, wave = 32 keys, streams Q/dO.
+//   S = Q K^T, dP = dO V^T, P = exp(S - lse), dS = P o (dP - delta),
+//   dV^T += dO^T P, dK^T += Q^T dS
+// (formulas: reference kernel/fused_mha_kernel.cu:598-603, 618-629, 653-656,
+// 697-712; key-block-parallel launch as at :908-915).
+// ---------------------------------------------------------------------------
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(kThreads, 1)
+fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
+                     const half_t* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ delta,
+                     half_t* __restrict__ dK, half_t* __restrict__ dV, int H, int N, float c, float scale) {
+  using G = TileGeom<D>;
+  __shared__ __attribute__((aligned(16))) char smem[4 * G::kTileBytes];  // Q0 dO0 Q1 dO1
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = lane & 31, hh = lane >> 5;
+  const int nblk = blockIdx.x;  // causal: low key blocks are the heavy ones and already come first
+  const int b = blockIdx.y / H, h = blockIdx.y % H;
+  const long rs = (long)H * D;
+  const long head_off = ((long)b * N * H + h) * D;
+  const half_t* Qb = Q + head_off;
+  const half_t* dOb = dO + head_off;
+  const float* lse_b = LSE + ((long)b * H + h) * N;
+  const float* delta_b = delta + ((long)b * H + h) * N;
+
+  const int n0 = nblk * kBlockRes;
+  const int k0w = n0 + wave * kResident;
+  const int ki = k0w + i;
+  const int krow = min(ki, N - 1);
+
+  h8 kf[G::kKSteps], vf[G::kKSteps];
+  {
+    const half_t* kp = K + head_off + (long)krow * rs + hh * 8;
+    const half_t* vp = V + head_off + (long)krow * rs + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+      kf[kk] = *reinterpret_cast<const h8*>(kp + kk * 16);
+      vf[kk] = *reinterpret_cast<const h8*>(vp + kk * 16);
+    }
+  }
+
+  const int nt = (N + kTile - 1) / kTile;
+  const int t_begin = CAUSAL ? n0 / kTile : 0;
+
+  const int lane_row_off = i * G::kRowBytes + hh * 16;
+  const int lane_tr_off = (4 * hh + ((lane & 15) >> 2)) * G::kRowBytes + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+
+  f16v dk[G::kDBlocks], dv[G::kDBlocks];
+#pragma unroll
+  for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
+
+  h8 qreg[G::kChunksPerThread], greg[G::kChunksPerThread];
+  if (t_begin < nt) {
+    tile_load<D>(Qb, rs, t_begin * kTile, N, qreg);
+    tile_load<D>(dOb, rs, t_begin * kTile, N, greg);
+    tile_store<D>(smem, qreg);
+    tile_store<D>(smem + G::kTileBytes, greg);
+  }
+  __syncthreads();
+
+  for (int qt = t_begin; qt < nt; ++qt) {
+    const int buf = (qt - t_begin) & 1;
+    const char* Ql = smem + buf * 2 * G::kTileBytes;
+    const char* Gl = Ql + G::kTileBytes;
+    const bool more = qt + 1 < nt;
+    if (more) {
+      tile_load<D>(Qb, rs, (qt + 1) * kTile, N, qreg);
+      tile_load<D>(dOb, rs, (qt + 1) * kTile, N, greg);
+    }
+    const int q0 = qt * kTile;
+    const bool active = !CAUSAL || q0 + kTile - 1 >= k0w;
+    if (active) {
+      const bool need_mask = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        f16v s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int kk = 0; kk < G::kKSteps; ++kk) {
+          s = mfma(read_rows<D>(Ql, rb, kk, lane_row_off), kf[kk], s);
+          dp = mfma(read_rows<D>(Gl, rb, kk, lane_row_off), vf[kk], dp);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int qg = q0 + rb * 32 + 8 * g + 4 * hh;  // 4 consecutive queries, multiple of 4
+          const int qld = min(qg, N - 4);
+          const f4v l4 = *reinterpret_cast<const f4v*>(lse_b + qld);
+          const f4v d4 = *reinterpret_cast<const f4v*>(delta_b + qld);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 4 * g + e;
+            float p = fast_exp2(fmaf(s[r], c, -l4[e] * kLog2e));
+            if (need_mask) {
+              int q = qg + e;
+              if ((CAUSAL && ki > q) || q >= N) p = 0.f;
+            }
+            s[r] = p;
+            dp[r] = p * (dp[r] - d4[e]);
+          }
+        }
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+          const h8 pf = pack8(s, cc * 8);
+          const h8 dsf = pack8(dp, cc * 8);
+          const int c16 = rb * 2 + cc;
+#pragma unroll
+          for (int db = 0; db < G::kDBlocks; ++db) {
+            dv[db] = mfma(read_cols<D>(Gl, c16, db, lane_tr_off), pf, dv[db]);
+            dk[db] = mfma(read_cols<D>(Ql, c16, db, lane_tr_off), dsf, dk[db]);
+          }
+        }
+      }
+    }
+    if (more) {
+      char* Qn = smem + (buf ^ 1) * 2 * G::kTileBytes;
+      tile_store<D>(Qn, qreg);
+      tile_store<D>(Qn + G::kTileBytes, greg);
+    }
+    __syncthreads();
+  }
+  store_resident<D>(dK + head_off, rs, ki, N, dk, scale, hh);
+  store_resident<D>(dV + head_off, rs, ki, N, dv, 1.f, hh);
+}
+
+// ---------------------------------------------------------------------------
+// Host side: validation and launches.
+// ---------------------------------------------------------------------------
+int check_shape(int batch, int head, int m, int n, int d) {
+  if (batch <= 0 || head <= 0 || n <= 0 || m != n || (n % 32) != 0) return FUSED_MHA_ERR_BAD_SHAPE;
+  if (d != 64 && d != 128) return FUSED_MHA_ERR_BAD_HEAD_DIM;
+  if ((long)batch * head > 65535) return FUSED_MHA_ERR_TOO_LARGE;
+  return FUSED_MHA_OK;
+}
+
+bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+template <int D, bool CAUSAL>
+int launch_forward(const void* q, const void* k, const void* v, void* o, void* lse, int batch, int head, int n,
+                   float scale, hipStream_t stream) {
+  dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
+  const float c = fabsf(scale) * kLog2e;
+  fmha_fwd_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+      (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, (float*)lse, head, n, c, scale < 0.f ? 1 : 0);
+  return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
+}
+
+template <int D, bool CAUSAL>
+int launch_backward(const void* q, const void* k, const void* v, const void* o, const void* d_o, const void* lse,
+                    float* delta, void* dq, void* dk, void* dv, int batch, int head, int n, float scale,
+                    hipStream_t stream) {
+  const long rows = (long)batch * n * head;
+  const long threads = rows * (D / 8);
+  fmha_bwd_delta_kernel<D><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(
+      (const half_t*)o, (const half_t*)d_o, delta, head, n, rows);
+  if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+  dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
+  const float c = scale * kLog2e;
+  fmha_bwd_dq_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+      (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
+      (half_t*)dq, head, n, c, scale);
+  if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+  fmha_bwd_dkdv_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+      (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
+      (half_t*)dk, (half_t*)dv, head, n, c, scale);
+  return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fused_mha_forward(const void* query_ptr, const void* key_ptr, const void* value_ptr, void* output_ptr,
+                      void* lse_ptr, int batch, int head, int m, int n, int d, float scale, int causal,
+                      void* stream) {
+  if (!query_ptr || !key_ptr || !value_ptr || !output_ptr || !lse_ptr) return FUSED_MHA_ERR_NULL_POINTER;
+  if (int rc = check_shape(batch, head, m, n, d)) return rc;
+  if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
+  if (misaligned(query_ptr) || misaligned(key_ptr) || misaligned(value_ptr) || misaligned(output_ptr) ||
+      misaligned(lse_ptr))
+    return FUSED_MHA_ERR_MISALIGNED;
+  hipStream_t s = (hipStream_t)stream;
+  if (d == 128) {
+    return causal ? launch_forward<128, true>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s)
+                  : launch_forward<128, false>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s);
+  }
+  return causal ? launch_forward<64, true>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s)
+                : launch_forward<64, false>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s);
+}
+
+size_t fused_mha_backward_workspace_bytes(int batch, int head, int n, int d) {
+  if (check_shape(batch, head, n, n, d) != FUSED_MHA_OK) return 0;
+  return (size_t)batch * head * n * sizeof(float);
+}
+
+int fused_mha_backward(const void* query_ptr, const void* key_ptr, const void* value_ptr, const void* output_ptr,
+                       const void* d_output_ptr, const void* lse_ptr, void* workspace, size_t workspace_bytes,
+                       void* d_query_ptr, void* d_key_ptr, void* d_value_ptr, int batch, int head, int m, int n,
+                       int d, float scale, int causal, void* stream) {
+  if (!query_ptr || !key_ptr || !value_ptr || !output_ptr || !d_output_ptr || !lse_ptr || !workspace ||
+      !d_query_ptr || !d_key_ptr || !d_value_ptr)
+    return FUSED_MHA_ERR_NULL_POINTER;
+  if (int rc = check_shape(batch, head, m, n, d)) return rc;
+  if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
+  if (workspace_bytes < fused_mha_backward_workspace_bytes(batch, head, n, d)) return FUSED_MHA_ERR_BAD_SHAPE;
+  if (misaligned(query_ptr) || misaligned(key_ptr) || misaligned(value_ptr) || misaligned(output_ptr) ||
+      misaligned(d_output_ptr) || misaligned(lse_ptr) || misaligned(workspace) || misaligned(d_query_ptr) ||
+      misaligned(d_key_ptr) || misaligned(d_value_ptr))
+    return FUSED_MHA_ERR_MISALIGNED;
+  hipStream_t s = (hipStream_t)stream;
+  float* delta = (float*)workspace;
+#define FMHA_BWD(DD, CC)                                                                                       \
+  launch_backward<DD, CC>(query_ptr, key_ptr, value_ptr, output_ptr, d_output_ptr, lse_ptr, delta, d_query_ptr, \
+                          d_key_ptr, d_value_ptr, batch, head, n, scale, s)
+  if (d == 128) return causal ? FMHA_BWD(128, true) : FMHA_BWD(128, false);
+  return causal ? FMHA_BWD(64, true) : FMHA_BWD(64, false);
+#undef FMHA_BWD
+}
+
+const char* fused_mha_error_string(int code) {
+  switch (code) {
+    case FUSED_MHA_OK: return "ok";
+    case FUSED_MHA_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case FUSED_MHA_ERR_BAD_SHAPE: return "bad shape: need batch, head, n > 0, m == n, n % 32 == 0 and a large enough workspace";
+    case FUSED_MHA_ERR_BAD_HEAD_DIM: return "head dimension must be 64 or 128";
+    case FUSED_MHA_ERR_MISALIGNED: return "a pointer is not 16-byte aligned";
+    case FUSED_MHA_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";
+    case FUSED_MHA_ERR_BAD_SCALE: return "scale must be finite";
+    case FUSED_MHA_ERR_TOO_LARGE: return "batch * head exceeds 65535";
+    default: return "unknown fused_mha error code";
+  }
+}
+
+}  // extern "C"

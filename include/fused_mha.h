@@ -1,0 +1,85 @@
+/*
+ * C ABI of the gfx950 fused multi-head attention launchers.
+ *
+ * These entry points take the place of the two launchers the reference
+ * declares in include/fused_mha.h:1-6 (defined at
+ * kernel/fused_mha_kernel.cu:891-916).  Plain pointers and sizes only: no
+ * torch types, so any host language can bind them (ctypes, cgo, JNI ...).
+ *
+ * Conventions shared by every entry point
+ *   - q, k, v, o, d_o, d_q, d_k, d_v: dense fp16 tensors of shape
+ *     (batch, n, head, d), element offset ((b*n + i)*head + h)*d + j
+ *     (reference: kernel/fused_mha_kernel.cu:57-59).
+ *   - lse: dense fp32 (batch, head, n): natural-log logsumexp of the scaled,
+ *     masked score row, i.e. max + ln(sum) of the two statistics the
+ *     reference stores separately (kernel/fused_mha_kernel.cu:298-303).
+ *   - m == n (self attention, reference: kernel/fused_mha_api.cpp:68-69),
+ *     n a multiple of 32 (reference: README.md:3), d is 64 or 128.
+ *   - causal != 0: key j is visible to query i iff j <= i
+ *     (reference: test.py:15-19).
+ *   - stream is a hipStream_t passed as void*; NULL is the default stream.
+ *     All work is enqueued asynchronously; nothing synchronises.
+ *   - All pointers are borrowed device pointers and must be 16-byte aligned.
+ *   - Return value: FUSED_MHA_OK (0) or a negative FUSED_MHA_ERR_* code.
+ *     Nothing is launched when an error is returned.
+ */
+#ifndef FUSED_MHA_H_
+#define FUSED_MHA_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FUSED_MHA_OK 0
+#define FUSED_MHA_ERR_NULL_POINTER (-1)   /* a required pointer is NULL            */
+#define FUSED_MHA_ERR_BAD_SHAPE (-2)      /* batch/head/n <= 0, m != n, n % 32 != 0 */
+#define FUSED_MHA_ERR_BAD_HEAD_DIM (-3)   /* d is neither 64 nor 128               */
+#define FUSED_MHA_ERR_MISALIGNED (-4)     /* a pointer is not 16-byte aligned      */
+#define FUSED_MHA_ERR_LAUNCH (-5)         /* the HIP runtime refused the launch    */
+#define FUSED_MHA_ERR_BAD_SCALE (-6)      /* scale is NaN or infinite              */
+#define FUSED_MHA_ERR_TOO_LARGE (-7)      /* batch*head exceeds the grid limit     */
+
+/*
+ * Forward: o = softmax(scale * q k^T  [+ causal mask]) v, lse = row logsumexp.
+ * Replaces fused_mha_forward (reference include/fused_mha.h:1-2); differs in
+ * writing one logsumexp tensor instead of max_ptr and sum_ptr, in returning an
+ * error code, and in accepting d = 64 as well as 128.
+ */
+int fused_mha_forward(const void *query_ptr, const void *key_ptr, const void *value_ptr,
+                      void *output_ptr, void *lse_ptr,
+                      int batch, int head, int m, int n, int d,
+                      float scale, int causal, void *stream);
+
+/*
+ * Bytes of device scratch fused_mha_backward needs for this problem size
+ * (holds delta = rowsum(d_o * o) in fp32, shape (batch, head, n)).
+ * Returns 0 for an invalid shape.  No counterpart in the reference, which
+ * receives delta from Python (flash_attn_interface.py:43-44).
+ */
+size_t fused_mha_backward_workspace_bytes(int batch, int head, int n, int d);
+
+/*
+ * Backward: d_q, d_k, d_v of the forward above, given d_o, the forward's
+ * output o and lse.  Replaces fused_mha_backward (reference
+ * include/fused_mha.h:4-6); differs in taking lse instead of max_ptr/sum_ptr,
+ * in computing delta itself into `workspace` (fp32 accumulation) instead of
+ * receiving a fp16 d_ptr, and in not requiring d_q to be zero-filled: every
+ * element of d_q, d_k and d_v is overwritten.
+ */
+int fused_mha_backward(const void *query_ptr, const void *key_ptr, const void *value_ptr,
+                       const void *output_ptr, const void *d_output_ptr, const void *lse_ptr,
+                       void *workspace, size_t workspace_bytes,
+                       void *d_query_ptr, void *d_key_ptr, void *d_value_ptr,
+                       int batch, int head, int m, int n, int d,
+                       float scale, int causal, void *stream);
+
+/* Static, human-readable text for a FUSED_MHA_* code. */
+const char *fused_mha_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FUSED_MHA_H_ */
