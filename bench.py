@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step is one forward + backward of the headline workload (B=2, H=32, N=4096,
+D=128, causal, fp16) through flash_attn_func(...).backward(dO): every kernel the
+autograd path launches is inside the timed region, inputs are resident in HBM.
+
+Prints ONE JSON line.  `value` is forward+backward TFLOP/s with the algorithmic
+FLOP count 3.5 * 4*B*H*N^2*D / 2 (causal); the forward alone, the per-kernel
+roofline of the slowest kernel, every other configuration, and a CPU baseline
+(the fp32 oracle on the host cores, a bounded sample) ride along.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "flash-attention-v100_amd"), os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_TFLOPS = 2516.6  # MI355X dense fp16 MFMA, vendor figure
+
+CONFIGS = [  # name, B, H, N, D, causal
+    ("plumbing_b1_h4_n128_d64", 1, 4, 128, 64, False),
+    ("bert_base_b16_h12_n512_d64", 16, 12, 512, 64, False),
+    ("gpt_causal_b4_h16_n1024_d64", 4, 16, 1024, 64, True),
+    ("llama7b_b2_h32_n4096_d128_causal", 2, 32, 4096, 128, True),
+    ("long_context_b1_h16_n16384_d128_causal", 1, 16, 16384, 128, True),
+]
+HEADLINE = 3
+
+
+def fwd_flops(B, H, N, D, causal):
+    f = 4.0 * B * H * N * N * D
+    return f * 0.5 if causal else f
+
+
+def time_ms(fn, steps, warmup):
+    """Device-event time per call on torch's current stream (the stream every
+    kernel here is launched on)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def make_device_inputs(B, H, N, D, seed=20):
+    import torch
+
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    return [torch.randn((B, N, H, D), generator=g, dtype=torch.float32).to(torch.float16).cuda() for _ in range(4)]
+
+
+def bench_config(B, H, N, D, causal, steps, warmup):
+    import torch
+    from flash_attn_v100 import flash_attn_func
+
+    q, k, v, do = make_device_inputs(B, H, N, D)
+    q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+    scale = 1.0 / math.sqrt(D)
+
+    def fwd():
+        with torch.no_grad():
+            flash_attn_func(q, k, v, scale, causal)
+
+    def fwd_bwd():
+        out = flash_attn_func(q, k, v, scale, causal)
+        out.backward(do)
+        q.grad = k.grad = v.grad = None
+
+    t_f = time_ms(fwd, steps, warmup)
+    t_fb = time_ms(fwd_bwd, steps, warmup)
+    ff = fwd_flops(B, H, N, D, causal)
+    return {"fwd_ms": t_f, "fwd_bwd_ms": t_fb, "fwd_tflops": ff / t_f / 1e9, "fwd_bwd_tflops": 3.5 * ff / t_fb / 1e9}
+
+
+def kernel_times(B, H, N, D, causal, steps, warmup):
+    """Average duration of each kernel, timed one by one through the C ABI."""
+    import torch
+    import abi
+
+    lib = abi.load()
+    q, k, v, do = make_device_inputs(B, H, N, D)
+    scale = 1.0 / math.sqrt(D)
+    out, lse = abi.forward(lib, q, k, v, scale, causal)
+    nbytes = lib.fused_mha_backward_workspace_bytes(B, H, N, D)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+    s = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+    c = int(causal)
+    calls = {
+        "fmha_fwd_kernel": lambda: lib.fused_mha_forward(p(q), p(k), p(v), p(out), p(lse), B, H, N, N, D, scale, c, s),
+        "fmha_bwd_delta_kernel": lambda: lib.fused_mha_backward_delta(p(out), p(do), p(ws), nbytes, B, H, N, D, s),
+        "fmha_bwd_dq_kernel": lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dq),
+                                                                 B, H, N, D, scale, c, s),
+        "fmha_bwd_dkdv_kernel": lambda: lib.fused_mha_backward_dkdv(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes,
+                                                                     p(dk), p(dv), B, H, N, D, scale, c, s),
+    }
+    return {name: time_ms(fn, steps, warmup) for name, fn in calls.items()}
+
+
+def cpu_baseline(B, H, N, D, causal, budget_s=12.0):
+    """The fp32 oracle (forward + analytic backward) on the host cores, over as
+    many (batch, head) slices of the headline workload as fit the time budget."""
+    import torch
+    from oracle import attention_oracle as ao
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    g = torch.Generator(device="cpu")
+    g.manual_seed(20)
+    q, k, v, do = (torch.randn((1, N, 1, D), generator=g).half() for _ in range(4))
+    scale = 1.0 / math.sqrt(D)
+    ao.attention_forward(q[:, :256], k[:, :256], v[:, :256], scale, causal)  # warm the thread pool
+    done, t0 = 0, time.perf_counter()
+    while done < B * H:
+        ao.attention_forward(q, k, v, scale, causal)
+        ao.attention_backward(q, k, v, do, scale, causal)
+        done += 1
+        if time.perf_counter() - t0 > budget_s:
+            break
+    dt = time.perf_counter() - t0
+    flops = 3.5 * fwd_flops(1, 1, N, D, causal) * done
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{done} of {B * H} (batch, head) slices of the headline workload, fwd+bwd, "
+                      f"fp32 torch on {cores} threads, {dt:.1f} s; dense N^2 work done, causal-halved FLOPs counted"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus)
+
+    import torch
+    from flash_attn_v100 import flash_attn_func
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    props = torch.cuda.get_device_properties(0)
+    clock_ghz = props.clock_rate / 1e6 if hasattr(props, "clock_rate") else 2.4
+    peak_check = props.multi_processor_count * 4 * 1024 * clock_ghz / 1e3  # CUs x SIMDs x flop/clk x GHz
+
+    name, B, H, N, D, causal = CONFIGS[HEADLINE]
+    q, k, v, do = make_device_inputs(B, H, N, D)
+    q.requires_grad_(), k.requires_grad_(), v.requires_grad_()
+    scale = 1.0 / math.sqrt(D)
+
+    def step():
+        out = flash_attn_func(q, k, v, scale, causal)
+        out.backward(do)
+        q.grad = k.grad = v.grad = None
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ff = fwd_flops(B, H, N, D, causal)
+    value = 3.5 * ff / ms / 1e9
+
+    def fwd_only():
+        with torch.no_grad():
+            flash_attn_func(q, k, v, scale, causal)
+
+    fwd_ms = time_ms(fwd_only, args.steps, args.warmup)
+    fwd_tflops = ff / fwd_ms / 1e9
+
+    # per-kernel durations and the roofline of the slowest kernel
+    kt = kernel_times(B, H, N, D, causal, args.steps, args.warmup)
+    # algorithmic FLOPs per launch: the GEMMs of the 5-GEMM backward / 2-GEMM forward
+    # count that each kernel produces (recomputed S and dP in the dQ pass are not counted)
+    alg = {"fmha_fwd_kernel": ff, "fmha_bwd_dkdv_kernel": 2.0 * ff, "fmha_bwd_dq_kernel": 0.5 * ff}
+    dominant = max(alg, key=lambda n: kt[n])
+    achieved = alg[dominant] / kt[dominant] / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(dominant)
+    roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / PEAK_TFLOPS, "traffic": traffic,
+                "kernel_ms": kt, "peak_check_tflops": peak_check}
+
+    others = {}
+    if not args.headline_only:
+        for cname, cB, cH, cN, cD, cc in CONFIGS:
+            r = bench_config(cB, cH, cN, cD, cc, max(5, args.steps // 2), max(3, args.warmup // 2))
+            r["fwd_frac_peak"] = r["fwd_tflops"] / PEAK_TFLOPS
+            r["fwd_bwd_frac_peak"] = r["fwd_bwd_tflops"] / PEAK_TFLOPS
+            others[cname] = {key: round(val, 5) for key, val in r.items()}
+
+    line = {
+        "metric": "fwd+bwd TFLOP/s, B2 H32 N4096 D128 causal fp16 (fwd alone in 'fwd')",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": name, "batch": B, "heads": H, "seq_len": N, "head_dim": D, "causal": causal},
+        "frac_of_peak": value / PEAK_TFLOPS,
+        "fwd": {"ms": fwd_ms, "tflops": fwd_tflops, "frac_of_peak": fwd_tflops / PEAK_TFLOPS},
+        "roofline": roofline,
+        "all_configs": others,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(B, H, N, D, causal)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

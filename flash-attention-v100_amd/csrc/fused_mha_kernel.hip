@@ -570,31 +570,64 @@ template <int D, bool CAUSAL>
 int launch_forward(const void* q, const void* k, const void* v, void* o, void* lse, int batch, int head, int n,
                    float scale, hipStream_t stream) {
   dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
-  const float c = fabsf(scale) * kLog2e;
+  // scale == 0 would turn the masked scores (-inf) into NaN when multiplied; a
+  // tiny positive factor gives the same uniform softmax and keeps -inf * c = -inf.
+  const float c = fmaxf(fabsf(scale) * kLog2e, 1e-30f);
   fmha_fwd_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
       (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, (float*)lse, head, n, c, scale < 0.f ? 1 : 0);
   return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
 }
 
+enum BwdPass { kPassDelta = 1, kPassDq = 2, kPassDkDv = 4, kPassAll = 7 };
+
 template <int D, bool CAUSAL>
-int launch_backward(const void* q, const void* k, const void* v, const void* o, const void* d_o, const void* lse,
-                    float* delta, void* dq, void* dk, void* dv, int batch, int head, int n, float scale,
-                    hipStream_t stream) {
-  const long rows = (long)batch * n * head;
-  const long threads = rows * (D / 8);
-  fmha_bwd_delta_kernel<D><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(
-      (const half_t*)o, (const half_t*)d_o, delta, head, n, rows);
-  if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+int launch_backward(int passes, const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                    const void* lse, float* delta, void* dq, void* dk, void* dv, int batch, int head, int n,
+                    float scale, hipStream_t stream) {
+  if (passes & kPassDelta) {
+    const long rows = (long)batch * n * head;
+    const long threads = rows * (D / 8);
+    fmha_bwd_delta_kernel<D><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(
+        (const half_t*)o, (const half_t*)d_o, delta, head, n, rows);
+    if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+  }
   dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
   const float c = scale * kLog2e;
-  fmha_bwd_dq_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
-      (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
-      (half_t*)dq, head, n, c, scale);
-  if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
-  fmha_bwd_dkdv_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
-      (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
-      (half_t*)dk, (half_t*)dv, head, n, c, scale);
-  return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
+  if (passes & kPassDq) {
+    fmha_bwd_dq_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
+        (half_t*)dq, head, n, c, scale);
+    if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+  }
+  if (passes & kPassDkDv) {
+    fmha_bwd_dkdv_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
+        (half_t*)dk, (half_t*)dv, head, n, c, scale);
+    if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+  }
+  return FUSED_MHA_OK;
+}
+
+int dispatch_backward(int passes, const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                      const void* lse, void* workspace, size_t workspace_bytes, void* dq, void* dk, void* dv,
+                      int batch, int head, int m, int n, int d, float scale, int causal, void* stream) {
+  const bool need_o = passes & kPassDelta, need_dq = passes & kPassDq, need_dkdv = passes & kPassDkDv;
+  if (!d_o || !workspace || (need_o && !o) || ((need_dq || need_dkdv) && (!q || !k || !v || !lse)) ||
+      (need_dq && !dq) || (need_dkdv && (!dk || !dv)))
+    return FUSED_MHA_ERR_NULL_POINTER;
+  if (int rc = check_shape(batch, head, m, n, d)) return rc;
+  if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
+  if (workspace_bytes < (size_t)batch * head * n * sizeof(float)) return FUSED_MHA_ERR_BAD_SHAPE;
+  if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(o) || misaligned(d_o) || misaligned(lse) ||
+      misaligned(workspace) || misaligned(dq) || misaligned(dk) || misaligned(dv))
+    return FUSED_MHA_ERR_MISALIGNED;
+  hipStream_t s = (hipStream_t)stream;
+  float* delta = (float*)workspace;
+#define FMHA_BWD(DD, CC) \
+  launch_backward<DD, CC>(passes, q, k, v, o, d_o, lse, delta, dq, dk, dv, batch, head, n, scale, s)
+  if (d == 128) return causal ? FMHA_BWD(128, true) : FMHA_BWD(128, false);
+  return causal ? FMHA_BWD(64, true) : FMHA_BWD(64, false);
+#undef FMHA_BWD
 }
 
 }  // namespace
@@ -628,24 +661,32 @@ int fused_mha_backward(const void* query_ptr, const void* key_ptr, const void* v
                        const void* d_output_ptr, const void* lse_ptr, void* workspace, size_t workspace_bytes,
                        void* d_query_ptr, void* d_key_ptr, void* d_value_ptr, int batch, int head, int m, int n,
                        int d, float scale, int causal, void* stream) {
-  if (!query_ptr || !key_ptr || !value_ptr || !output_ptr || !d_output_ptr || !lse_ptr || !workspace ||
-      !d_query_ptr || !d_key_ptr || !d_value_ptr)
-    return FUSED_MHA_ERR_NULL_POINTER;
-  if (int rc = check_shape(batch, head, m, n, d)) return rc;
-  if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
-  if (workspace_bytes < fused_mha_backward_workspace_bytes(batch, head, n, d)) return FUSED_MHA_ERR_BAD_SHAPE;
-  if (misaligned(query_ptr) || misaligned(key_ptr) || misaligned(value_ptr) || misaligned(output_ptr) ||
-      misaligned(d_output_ptr) || misaligned(lse_ptr) || misaligned(workspace) || misaligned(d_query_ptr) ||
-      misaligned(d_key_ptr) || misaligned(d_value_ptr))
-    return FUSED_MHA_ERR_MISALIGNED;
-  hipStream_t s = (hipStream_t)stream;
-  float* delta = (float*)workspace;
-#define FMHA_BWD(DD, CC)                                                                                       \
-  launch_backward<DD, CC>(query_ptr, key_ptr, value_ptr, output_ptr, d_output_ptr, lse_ptr, delta, d_query_ptr, \
-                          d_key_ptr, d_value_ptr, batch, head, n, scale, s)
-  if (d == 128) return causal ? FMHA_BWD(128, true) : FMHA_BWD(128, false);
-  return causal ? FMHA_BWD(64, true) : FMHA_BWD(64, false);
-#undef FMHA_BWD
+  return dispatch_backward(kPassAll, query_ptr, key_ptr, value_ptr, output_ptr, d_output_ptr, lse_ptr, workspace,
+                           workspace_bytes, d_query_ptr, d_key_ptr, d_value_ptr, batch, head, m, n, d, scale, causal,
+                           stream);
+}
+
+int fused_mha_backward_delta(const void* output_ptr, const void* d_output_ptr, void* workspace,
+                             size_t workspace_bytes, int batch, int head, int n, int d, void* stream) {
+  return dispatch_backward(kPassDelta, nullptr, nullptr, nullptr, output_ptr, d_output_ptr, nullptr, workspace,
+                           workspace_bytes, nullptr, nullptr, nullptr, batch, head, n, n, d, 1.f, 0, stream);
+}
+
+int fused_mha_backward_dq(const void* query_ptr, const void* key_ptr, const void* value_ptr,
+                          const void* d_output_ptr, const void* lse_ptr, void* workspace, size_t workspace_bytes,
+                          void* d_query_ptr, int batch, int head, int n, int d, float scale, int causal,
+                          void* stream) {
+  return dispatch_backward(kPassDq, query_ptr, key_ptr, value_ptr, nullptr, d_output_ptr, lse_ptr, workspace,
+                           workspace_bytes, d_query_ptr, nullptr, nullptr, batch, head, n, n, d, scale, causal, stream);
+}
+
+int fused_mha_backward_dkdv(const void* query_ptr, const void* key_ptr, const void* value_ptr,
+                            const void* d_output_ptr, const void* lse_ptr, void* workspace, size_t workspace_bytes,
+                            void* d_key_ptr, void* d_value_ptr, int batch, int head, int n, int d, float scale,
+                            int causal, void* stream) {
+  return dispatch_backward(kPassDkDv, query_ptr, key_ptr, value_ptr, nullptr, d_output_ptr, lse_ptr, workspace,
+                           workspace_bytes, nullptr, d_key_ptr, d_value_ptr, batch, head, n, n, d, scale, causal,
+                           stream);
 }
 
 const char* fused_mha_error_string(int code) {

@@ -75,6 +75,30 @@ int fused_mha_backward(const void *query_ptr, const void *key_ptr, const void *v
                        int batch, int head, int m, int n, int d,
                        float scale, int causal, void *stream);
 
+/*
+ * The three passes fused_mha_backward enqueues, one entry point each, so a
+ * caller can time them separately or put the dQ pass and the dK/dV pass (which
+ * are independent of each other, both depend on the delta pass) on different
+ * streams.  Same conventions and workspace as fused_mha_backward.  No
+ * counterpart in the reference, whose backward is a single kernel
+ * (kernel/fused_mha_kernel.cu:904-916).
+ *   delta : workspace[b][h][i] = sum_j d_o[b][i][h][j] * o[b][i][h][j]  (fp32)
+ *   dq    : d_q, streaming key/value tiles per block of 128 queries
+ *   dkdv  : d_k and d_v, streaming query/d_o tiles per block of 128 keys
+ */
+int fused_mha_backward_delta(const void *output_ptr, const void *d_output_ptr,
+                             void *workspace, size_t workspace_bytes,
+                             int batch, int head, int n, int d, void *stream);
+int fused_mha_backward_dq(const void *query_ptr, const void *key_ptr, const void *value_ptr,
+                          const void *d_output_ptr, const void *lse_ptr,
+                          void *workspace, size_t workspace_bytes, void *d_query_ptr,
+                          int batch, int head, int n, int d, float scale, int causal, void *stream);
+int fused_mha_backward_dkdv(const void *query_ptr, const void *key_ptr, const void *value_ptr,
+                            const void *d_output_ptr, const void *lse_ptr,
+                            void *workspace, size_t workspace_bytes,
+                            void *d_key_ptr, void *d_value_ptr,
+                            int batch, int head, int n, int d, float scale, int causal, void *stream);
+
 /* Static, human-readable text for a FUSED_MHA_* code. */
 const char *fused_mha_error_string(int code);
 

@@ -1,0 +1,121 @@
+"""CPU tests of the host side: the C ABI library loads and exports what the
+header declares, argument validation returns the documented codes before any
+launch, and the extension raises RuntimeError like the reference's TORCH_CHECKs
+(kernel/fused_mha_api.cpp:25-47).  No compute call is made here."""
+import ctypes
+import inspect
+
+import pytest
+import torch
+
+import abi
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return abi.load()
+
+
+def test_exports_every_declared_symbol(lib):
+    names = abi.declared_symbols()
+    assert names == sorted(["fused_mha_forward", "fused_mha_backward", "fused_mha_backward_workspace_bytes",
+                            "fused_mha_backward_delta", "fused_mha_backward_dq", "fused_mha_backward_dkdv",
+                            "fused_mha_error_string"])
+    for name in names:
+        assert hasattr(lib, name), name
+
+
+def test_error_strings(lib):
+    seen = set()
+    for code in range(0, -8, -1):
+        text = lib.fused_mha_error_string(code).decode()
+        assert text and text not in seen
+        seen.add(text)
+    assert b"unknown" in lib.fused_mha_error_string(-99)
+
+
+def test_workspace_bytes(lib):
+    assert lib.fused_mha_backward_workspace_bytes(2, 32, 4096, 128) == 2 * 32 * 4096 * 4
+    assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 64) == 4 * 128 * 4
+    assert lib.fused_mha_backward_workspace_bytes(1, 4, 100, 64) == 0
+    assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 96) == 0
+
+
+def test_forward_validation_codes(lib):
+    p = 0x1000  # never dereferenced: every call below is rejected before a launch
+    f = lib.fused_mha_forward
+    assert f(None, p, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+    assert f(p, p, p, p, None, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+    assert f(p, p, p, p, p, 0, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE
+    assert f(p, p, p, p, p, 1, 1, 48, 48, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE      # n % 32
+    assert f(p, p, p, p, p, 1, 1, 32, 64, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE      # m != n
+    assert f(p, p, p, p, p, 1, 1, 32, 32, 96, 1.0, 0, None) == abi.ERR_BAD_HEAD_DIM
+    assert f(p, p, p, p, p, 1, 1, 32, 32, 64, float("nan"), 0, None) == abi.ERR_BAD_SCALE
+    assert f(p, p, p, p, p, 1, 1, 32, 32, 64, float("inf"), 0, None) == abi.ERR_BAD_SCALE
+    assert f(p + 2, p, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_MISALIGNED
+    assert f(p, p, p, p, p, 4096, 32, 32, 32, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
+
+
+def test_backward_validation_codes(lib):
+    p = 0x1000
+    b = lib.fused_mha_backward
+    ws = 1 * 1 * 32 * 4
+    assert b(p, p, p, p, p, p, None, ws, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+    assert b(p, p, p, p, p, p, p, ws, p, p, None, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+    assert b(p, p, p, p, p, p, p, ws - 1, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE
+    assert b(p, p, p, p, p, p, p, ws, p, p, p, 1, 1, 40, 40, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE
+    assert b(p, p, p, p, p, p, p, ws, p, p, p, 1, 1, 32, 32, 32, 1.0, 0, None) == abi.ERR_BAD_HEAD_DIM
+    assert b(p, p, p, p, p, p, p, ws, p, p + 8, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_MISALIGNED
+    assert lib.fused_mha_backward_delta(p, None, p, ws, 1, 1, 32, 64, None) == abi.ERR_NULL_POINTER
+    assert lib.fused_mha_backward_dq(p, p, p, p, p, p, ws, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+    assert lib.fused_mha_backward_dkdv(p, p, p, p, p, p, ws, p, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+
+
+def test_python_api_signature():
+    import flash_attn_v100
+    from flash_attn_v100 import flash_attn_func
+    from flash_attn_v100.flash_attn_interface import FlashAttnFunc
+
+    assert flash_attn_v100.__version__
+    params = inspect.signature(flash_attn_func).parameters
+    # reference flash_attn_interface.py:101-107
+    assert list(params) == ["q", "k", "v", "softmax_scale", "causal"]
+    assert params["softmax_scale"].default is None and params["causal"].default is False
+    assert issubclass(FlashAttnFunc, torch.autograd.Function)
+
+
+def test_extension_checks_raise_runtime_error():
+    import flash_attn_v100_cuda as ext
+
+    def t(*shape, dtype=torch.float16):
+        return torch.zeros(shape, dtype=dtype)
+
+    ok = t(1, 32, 2, 64)
+    cases = [
+        ((t(1, 32, 2, 64, dtype=torch.float32), ok, ok), "fp16"),
+        ((ok, t(1, 32, 2, 64, dtype=torch.bfloat16), ok), "same dtype"),
+        ((t(32, 2, 64), ok, ok), "4 dimensions"),
+        ((t(1, 32, 2, 96), t(1, 32, 2, 96), t(1, 32, 2, 96)), "head dimension"),
+        ((t(1, 48, 2, 64), t(1, 48, 2, 64), t(1, 48, 2, 64)), "multiple of 32"),
+        ((ok, t(1, 64, 2, 64), ok), "must have shape"),
+        ((t(1, 32, 2, 128)[..., ::2], ok, ok), "contiguous last dimension"),
+        ((ok, ok, ok), "must be on the GPU"),
+    ]
+    for (q, k, v), msg in cases:
+        with pytest.raises(RuntimeError, match=msg):
+            ext.fwd(q, k, v, None, 0.125, False)
+    lse = torch.zeros(1, 2, 32)
+    with pytest.raises(RuntimeError, match="must be on the GPU"):
+        ext.bwd(ok, ok, ok, ok, ok, lse, None, None, None, 0.125, True)
+    with pytest.raises(RuntimeError, match="lse must be fp32"):
+        ext.bwd(ok, ok, ok, ok, ok, lse.half(), None, None, None, 0.125, True)
+    with pytest.raises(RuntimeError, match="must have shape"):
+        ext.bwd(ok, ok, ok, ok, ok, torch.zeros(1, 32, 2), None, None, None, 0.125, True)
+
+
+def test_python_api_rejects_cpu_tensors():
+    from flash_attn_v100 import flash_attn_func
+
+    q = torch.zeros(1, 32, 2, 64, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="must be on the GPU"):
+        flash_attn_func(q, q, q, None, True)
