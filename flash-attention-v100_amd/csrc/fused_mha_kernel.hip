@@ -154,20 +154,123 @@ __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long r
 }
 
 // ---------------------------------------------------------------------------
-// Forward.  Block = 128 queries, wave = 32 queries, streams K/V tiles of 64.
+// Streaming of 64-row tiles, global -> registers -> LDS, with per-thread
+// offsets computed once.  PAD is the padding of an LDS row in bytes: 16 makes
+// the 128-bit row reads conflict-free, 32 the transposed 64-bit reads.
 // ---------------------------------------------------------------------------
+template <int D, int PAD>
+struct TileStream {
+  static constexpr int kRowBytes = D * 2 + PAD;
+  static constexpr int kTileBytes = kTile * kRowBytes;
+  static constexpr int kCPT = TileGeom<D>::kChunksPerThread;
+  int goff[kCPT];  // element offset of this thread's chunks inside a full tile
+  int loff[kCPT];  // byte offset inside the LDS tile
+  int row[kCPT];
+  int col[kCPT];
+
+  __device__ __forceinline__ void init(int row_stride) {
+#pragma unroll
+    for (int i = 0; i < kCPT; ++i) {
+      int ch = threadIdx.x + kThreads * i;
+      row[i] = ch / TileGeom<D>::kChunksPerRow;
+      col[i] = (ch % TileGeom<D>::kChunksPerRow) * 8;
+      goff[i] = row[i] * row_stride + col[i];
+      loff[i] = row[i] * kRowBytes + col[i] * 2;
+    }
+  }
+  // `base` points at row 0 of the (batch, head) slice; rows past n-1 are clamped.
+  __device__ __forceinline__ void load(const half_t* __restrict__ base, int row_stride, int row0, int n,
+                                       h8 (&regs)[kCPT]) const {
+    const half_t* tile = base + (long)row0 * row_stride;  // wave-uniform
+    if (row0 + kTile <= n) {
+#pragma unroll
+      for (int i = 0; i < kCPT; ++i) regs[i] = *reinterpret_cast<const h8*>(tile + goff[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kCPT; ++i) {
+        int r = min(row0 + row[i], n - 1);
+        regs[i] = *reinterpret_cast<const h8*>(base + (long)r * row_stride + col[i]);
+      }
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, const h8 (&regs)[kCPT]) const {
+#pragma unroll
+    for (int i = 0; i < kCPT; ++i) *reinterpret_cast<h8*>(lds + loff[i]) = regs[i];
+  }
+};
+
+// Lane-constant byte offsets of the two LDS read patterns.
+template <int ROWB>
+__device__ __forceinline__ int lane_rows_off(int lane) { return (lane & 31) * ROWB + (lane >> 5) * 16; }
+template <int ROWB>
+__device__ __forceinline__ int lane_cols_off(int lane) {
+  return (4 * (lane >> 5) + ((lane & 15) >> 2)) * ROWB + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+}
+// A operand, rows = 32 streamed positions of row-block rb, k = features of k-step kk.
+template <int ROWB>
+__device__ __forceinline__ h8 lds_rows(const char* lds, int rb, int kk, int lane_off) {
+  return *reinterpret_cast<const h8*>(lds + lane_off + rb * 32 * ROWB + kk * 32);
+}
+// A operand, rows = 32 features of block db, k = streamed positions of chunk c16
+// in accumulator order (k index 8*hh + j <-> row 16*c16 + 8*(j/4) + 4*hh + j%4).
+template <int ROWB>
+__device__ __forceinline__ h8 lds_cols(const char* lds, int c16, int db, int lane_off) {
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const char* p = lds + lane_off + c16 * 16 * ROWB + db * 64;
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p));
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + 8 * ROWB));
+  return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// Sum of the 8 halves of x added to acc, two at a time (v_dot2_f32_f16).
+__device__ __forceinline__ float add_halves(h8 x, float acc) {
+  const h2 ones = {(half_t)1.f, (half_t)1.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    h2 pr = {x[2 * j], x[2 * j + 1]};
+    acc = __builtin_amdgcn_fdot2(pr, ones, acc, false);
+  }
+  return acc;
+}
+
+// Work-group id -> (batch*head slice, block inside the slice).  Consecutive
+// work-group ids go round-robin over the 8 XCDs, each with a private L2; the
+// remap hands every XCD whole (batch, head) slices, so the blocks that stream
+// the same K/V (or Q/dO) rows share one L2.
+__device__ __forceinline__ void slice_and_block(int blocks_per_slice, int& slice, int& blk) {
+  const int lin = blockIdx.x, total = gridDim.x;
+  int virt = lin;
+  if ((total & 7) == 0) virt = (lin & 7) * (total >> 3) + (lin >> 3);
+  slice = virt / blocks_per_slice;
+  blk = virt - slice * blocks_per_slice;
+}
+
+// ---------------------------------------------------------------------------
+// Forward.  Block = 128 queries, wave = 32 queries, streams K/V tiles of 64.
+// Online softmax as in reference kernel/fused_mha_kernel.cu:159-181, except
+// that the running max is only raised (and O, l rescaled) when it grew by more
+// than kRescaleLog2 in the exp2 domain, which is rare after the first tiles;
+// probabilities then stay below 2^kRescaleLog2 and the final O/l is unchanged.
+// ---------------------------------------------------------------------------
+constexpr float kRescaleLog2 = 8.f;
+
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(kThreads, 2)
 fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-                half_t* __restrict__ O, float* __restrict__ LSE, int H, int N, float c, int negate_q) {
+                half_t* __restrict__ O, float* __restrict__ LSE, int H, int N, int nmb, float c, int negate_q) {
   using G = TileGeom<D>;
-  __shared__ __attribute__((aligned(16))) char smem[4 * G::kTileBytes];  // K0 V0 K1 V1
+  using KS = TileStream<D, 16>;
+  using VS = TileStream<D, 32>;
+  constexpr int kBuf = KS::kTileBytes + VS::kTileBytes;
+  __shared__ __attribute__((aligned(16))) char smem[2 * kBuf];  // {K, V} x 2
 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int i = lane & 31, hh = lane >> 5;
-  const int mblk = CAUSAL ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;  // heavy blocks first
-  const int b = blockIdx.y / H, h = blockIdx.y % H;
-  const long rs = (long)H * D;
+  int bh, mb;
+  slice_and_block(nmb, bh, mb);
+  const int mblk = CAUSAL ? nmb - 1 - mb : mb;  // heavy blocks first
+  const int b = bh / H, h = bh - b * H;
+  const int rs = H * D;
   const long head_off = ((long)b * N * H + h) * D;
   const half_t* Qb = Q + head_off;
   const half_t* Kb = K + head_off;
@@ -190,8 +293,8 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   int nt = (N + kTile - 1) / kTile;
   if (CAUSAL) nt = min(nt, (min(m0 + kBlockRes, N) - 1) / kTile + 1);
 
-  const int lane_row_off = i * G::kRowBytes + hh * 16;
-  const int lane_tr_off = (4 * hh + ((lane & 15) >> 2)) * G::kRowBytes + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  const int k_off = lane_rows_off<KS::kRowBytes>(lane);
+  const int v_off = lane_cols_off<VS::kRowBytes>(lane);
 
   f16v o[G::kDBlocks];
 #pragma unroll
@@ -200,20 +303,24 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
     for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  h8 kreg[G::kChunksPerThread], vreg[G::kChunksPerThread];
-  tile_load<D>(Kb, rs, 0, N, kreg);
-  tile_load<D>(Vb, rs, 0, N, vreg);
-  tile_store<D>(smem, kreg);
-  tile_store<D>(smem + G::kTileBytes, vreg);
+  KS ks;
+  VS vs;
+  ks.init(rs);
+  vs.init(rs);
+  h8 kreg[KS::kCPT], vreg[VS::kCPT];
+  ks.load(Kb, rs, 0, N, kreg);
+  vs.load(Vb, rs, 0, N, vreg);
+  ks.store(smem, kreg);
+  vs.store(smem + KS::kTileBytes, vreg);
   __syncthreads();
 
   for (int kt = 0; kt < nt; ++kt) {
-    const char* Kl = smem + (kt & 1) * 2 * G::kTileBytes;
-    const char* Vl = Kl + G::kTileBytes;
+    const char* Kl = smem + (kt & 1) * kBuf;
+    const char* Vl = Kl + KS::kTileBytes;
     const bool more = kt + 1 < nt;
     if (more) {
-      tile_load<D>(Kb, rs, (kt + 1) * kTile, N, kreg);
-      tile_load<D>(Vb, rs, (kt + 1) * kTile, N, vreg);
+      ks.load(Kb, rs, (kt + 1) * kTile, N, kreg);
+      vs.load(Vb, rs, (kt + 1) * kTile, N, vreg);
     }
     const int key0 = kt * kTile;
     const bool active = !CAUSAL || key0 <= q0w + kResident - 1;
@@ -226,7 +333,7 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 #pragma unroll
       for (int kk = 0; kk < G::kKSteps; ++kk) {
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(read_rows<D>(Kl, rb, kk, lane_row_off), qf[kk], s[rb]);
+        for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(lds_rows<KS::kRowBytes>(Kl, rb, kk, k_off), qf[kk], s[rb]);
       }
       const bool need_mask = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
       if (need_mask) {
@@ -245,36 +352,33 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[rb][r]);
       mx = fmaxf(mx, other_half(mx));
       const float m_new = fmaxf(m_run, mx);
-      const float alpha = fast_exp2((m_run - m_new) * c);
-      const float mc = m_new * c;
-      m_run = m_new;
-      float rowsum = 0.f;
+      if (__builtin_amdgcn_ballot_w64((m_new - m_run) * c > kRescaleLog2) != 0) {
+        const float alpha = fast_exp2((m_run - m_new) * c);
+        m_run = m_new;
+        l_run *= alpha;
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
+        for (int db = 0; db < G::kDBlocks; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float p = fast_exp2(fmaf(s[rb][r], c, -mc));
-          s[rb][r] = p;
-          rowsum += p;
-        }
-      l_run = l_run * alpha + rowsum;
-#pragma unroll
-      for (int db = 0; db < G::kDBlocks; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+          for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+      }
+      const float mc = m_run * c;
       h8 pf[4];
-#pragma unroll
-      for (int c16 = 0; c16 < 4; ++c16) pf[c16] = pack8(s[c16 >> 1], (c16 & 1) * 8);
 #pragma unroll
       for (int c16 = 0; c16 < 4; ++c16) {
 #pragma unroll
-        for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(read_cols<D>(Vl, c16, db, lane_tr_off), pf[c16], o[db]);
+        for (int j = 0; j < 8; ++j) pf[c16][j] = (half_t)fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + j], c, -mc));
+        l_run = add_halves(pf[c16], l_run);
+      }
+#pragma unroll
+      for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+        for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(lds_cols<VS::kRowBytes>(Vl, c16, db, v_off), pf[c16], o[db]);
       }
     }
     if (more) {
-      char* Kn = smem + ((kt + 1) & 1) * 2 * G::kTileBytes;
-      tile_store<D>(Kn, kreg);
-      tile_store<D>(Kn + G::kTileBytes, vreg);
+      char* Kn = smem + ((kt + 1) & 1) * kBuf;
+      ks.store(Kn, kreg);
+      vs.store(Kn + KS::kTileBytes, vreg);
     }
     __syncthreads();
   }
@@ -569,12 +673,13 @@ bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) !
 template <int D, bool CAUSAL>
 int launch_forward(const void* q, const void* k, const void* v, void* o, void* lse, int batch, int head, int n,
                    float scale, hipStream_t stream) {
-  dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
+  const int nmb = (n + kBlockRes - 1) / kBlockRes;
+  dim3 grid(nmb * batch * head);
   // scale == 0 would turn the masked scores (-inf) into NaN when multiplied; a
   // tiny positive factor gives the same uniform softmax and keeps -inf * c = -inf.
   const float c = fmaxf(fabsf(scale) * kLog2e, 1e-30f);
   fmha_fwd_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
-      (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, (float*)lse, head, n, c, scale < 0.f ? 1 : 0);
+      (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, (float*)lse, head, n, nmb, c, scale < 0.f ? 1 : 0);
   return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
 }
 
