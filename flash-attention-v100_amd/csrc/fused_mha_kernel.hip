@@ -246,25 +246,152 @@ __device__ __forceinline__ void slice_and_block(int blocks_per_slice, int& slice
 }
 
 // ---------------------------------------------------------------------------
-// Forward.  Block = 128 queries, wave = 32 queries, streams K/V tiles of 64.
+// 64-row tiles copied global -> LDS by global_load_lds_dwordx4 (no registers in
+// between).  One wave-level instruction moves 1 KiB: 16 rows x 64 bytes, every
+// 4 lanes reading one 64-byte row segment.  The tile is an array of such 1 KiB
+// blocks, block (R, C) = rows 16R..16R+15, bytes 64C..64C+63 of each row.
+// Inside a block the 16-byte chunk c4 of row r16 sits at
+//     r16 * 64 + ((c4 ^ (r16 >> 2)) * 16),
+// which makes both read patterns below bank-conflict free without padding:
+//   rows:  16 lanes read the same chunk of 16 consecutive rows  (128-bit reads)
+//   cols:  16 lanes read 4 rows x 32 bytes, transposed         (ds_read_b64_tr_b16)
+// ---------------------------------------------------------------------------
+template <int D>
+struct SwzTile {
+  static constexpr int kNC = D / 32;              // 64-byte column groups per row
+  static constexpr int kBytes = kTile * D * 2;
+  static constexpr int kInstrs = 4 * kNC;         // 1 KiB copies per tile
+  __host__ __device__ static constexpr int block_off(int R, int C) { return (R * kNC + C) * 1024; }
+};
+
+// Per-lane source of copy instruction t (block R = t / kNC, C = t % kNC):
+// byte offset from the tile's first row, and the row inside the tile.
+template <int D>
+__device__ __forceinline__ void copy_src(int t, int lane, int row_stride, int& row, int& goff) {
+  const int R = t / SwzTile<D>::kNC, C = t % SwzTile<D>::kNC;
+  const int r16 = lane >> 2, pos = lane & 3;
+  const int c4 = pos ^ (r16 >> 2);
+  row = 16 * R + r16;
+  goff = (row * row_stride + (4 * C + c4) * 8) * 2;  // bytes
+}
+
+// One 1 KiB copy: lane l fetches 16 bytes at tile_base + voff and they land in
+// LDS at lds_block + 16 * l.  Written as inline asm on purpose: the compiler's
+// wait-count insertion then knows nothing of the copy, so it cannot make later
+// LDS reads wait for it (it cannot tell the ring slots apart and would wait for
+// every copy in flight); the waits for these copies are the explicit wait_vm<>
+// calls in the kernels.  tile_base and lds_block must be wave-uniform.
+__device__ __forceinline__ void copy16(const half_t* tile_base, int voff, char* lds_block) {
+  const unsigned lds_addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds_block;
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(voff), "s"(tile_base), "s"(lds_addr)
+      : "memory");
+}
+
+// rows pattern: lane (i, hh) reads chunk 2*kk + hh of row rb*32 + i.
+// Two lane offsets (kk even / odd); the rest is an immediate.
+template <int D>
+__device__ __forceinline__ void swz_rows_off(int lane, int (&off)[2]) {
+  const int i = lane & 31, hh = lane >> 5, r16 = i & 15, g = r16 >> 2;
+  const int base = (i >> 4) * SwzTile<D>::kNC * 1024 + r16 * 64;
+  off[0] = base + ((hh ^ g) * 16);
+  off[1] = base + (((2 + hh) ^ g) * 16);
+}
+template <int D>
+__device__ __forceinline__ h8 swz_rows(const char* tile, int rb, int kk, const int (&off)[2]) {
+  return *reinterpret_cast<const h8*>(tile + off[kk & 1] + SwzTile<D>::block_off(2 * rb, kk >> 1));
+}
+// cols pattern: MFMA A operand, rows = features db*32 + (lane & 31), k = streamed
+// rows of chunk c16 in accumulator order.  Two lane offsets (rows +0 / +8).
+template <int D>
+__device__ __forceinline__ void swz_cols_off(int lane, int (&off)[2]) {
+  const int L = lane & 15, half = (lane >> 4) & 1, hh = lane >> 5;
+  const int c4 = 2 * half + ((L & 3) >> 1);
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int r16 = 8 * e + 4 * hh + (L >> 2);
+    off[e] = r16 * 64 + ((c4 ^ (r16 >> 2)) * 16) + (L & 1) * 8;
+  }
+}
+template <int D>
+__device__ __forceinline__ h8 swz_cols(const char* tile, int c16, int db, const int (&off)[2]) {
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const char* p = tile + SwzTile<D>::block_off(c16, db);
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + off[0]));
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + off[1]));
+  return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// s_waitcnt vmcnt(N) with the other counters left alone.  Issued through the
+// builtin (not inline asm) so that the compiler's wait-count bookkeeping sees it.
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+  static_assert(N >= 0 && N < 16, "vmcnt immediate");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+}
+__device__ __forceinline__ void block_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads have landed
+  asm volatile("" ::: "memory");       // keep LDS accesses on their side of the barrier
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+template <int V>
+struct IntTag { static constexpr int value = V; };
+
+// ---------------------------------------------------------------------------
+// Forward.  Block = 8 waves = 256 queries, wave = 32 queries; K/V tiles of 64
+// keys stream through a 3-slot LDS ring, copied asynchronously two tiles ahead.
+//
 // Online softmax as in reference kernel/fused_mha_kernel.cu:159-181, except
 // that the running max is only raised (and O, l rescaled) when it grew by more
 // than kRescaleLog2 in the exp2 domain, which is rare after the first tiles;
 // probabilities then stay below 2^kRescaleLog2 and the final O/l is unchanged.
+//
+// The two waves that share a SIMD (w and w+4) run the same three steps per
+// tile, scores (MFMA), softmax (VALU), accumulate (MFMA), in rotated order:
+// waves 0-3 do  accumulate(j-1), scores(j), softmax(j)  in iteration j, waves
+// 4-7 do  softmax(j-1), accumulate(j-1), scores(j).  Both need exactly K(j)
+// and V(j-1) in iteration j, so one barrier per iteration is enough, and one
+// wave's MFMA stretch coincides with the other's VALU stretch.
 // ---------------------------------------------------------------------------
 constexpr float kRescaleLog2 = 8.f;
+constexpr int kFwdWaves = 8;
+constexpr int kFwdThreads = kFwdWaves * 64;
+constexpr int kFwdBlockQ = kFwdWaves * kResident;
+constexpr int kRing = 3;
 
 template <int D, bool CAUSAL>
-__global__ void __launch_bounds__(kThreads, 2)
+__global__ void __launch_bounds__(kFwdThreads, 1)
 fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
                 half_t* __restrict__ O, float* __restrict__ LSE, int H, int N, int nmb, float c, int negate_q) {
   using G = TileGeom<D>;
-  using KS = TileStream<D, 16>;
-  using VS = TileStream<D, 32>;
-  constexpr int kBuf = KS::kTileBytes + VS::kTileBytes;
-  __shared__ __attribute__((aligned(16))) char smem[2 * kBuf];  // {K, V} x 2
+  using T = SwzTile<D>;
+  constexpr int kIPW = T::kInstrs / kFwdWaves;  // copy instructions per wave per tile
+  // Ring slots are separate arrays, indexed with compile-time constants only, so
+  // the compiler can tell which slot an asynchronous copy writes and does not
+  // make LDS reads of the other slots wait for copies still in flight.
+  static_assert(kRing == 3, "the main loop is unrolled for three slots");
+  __shared__ __attribute__((aligned(1024))) char k_slot0[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char k_slot1[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char k_slot2[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char v_slot0[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char v_slot1[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char v_slot2[T::kBytes];
+  auto k_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
+    constexpr int S = decltype(tag)::value % kRing;
+    return S == 0 ? k_slot0 : S == 1 ? k_slot1 : k_slot2;
+  };
+  auto v_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
+    constexpr int S = decltype(tag)::value % kRing;
+    return S == 0 ? v_slot0 : S == 1 ? v_slot1 : v_slot2;
+  };
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 31, hh = lane >> 5;
   int bh, mb;
   slice_and_block(nmb, bh, mb);
@@ -276,9 +403,45 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   const half_t* Kb = K + head_off;
   const half_t* Vb = V + head_off;
 
-  const int m0 = mblk * kBlockRes;
+  const int m0 = mblk * kFwdBlockQ;
   const int q0w = m0 + wave * kResident;
   const int qi = q0w + i;
+
+  // nt: tiles the block streams; ntw: tiles this wave has unmasked keys in.
+  int nt = (N + kTile - 1) / kTile;
+  int ntw = nt;
+  if (CAUSAL) {
+    nt = min(nt, (min(m0 + kFwdBlockQ, N) - 1) / kTile + 1);
+    ntw = min(nt, (min(q0w + kResident, N) - 1) / kTile + 1);
+    if (q0w >= N) ntw = 0;
+  }
+
+  // this wave's share of every tile copy
+  int c_row[kIPW], c_goff[kIPW], c_blk[kIPW];
+#pragma unroll
+  for (int u = 0; u < kIPW; ++u) {
+    const int t = wave * kIPW + u;
+    copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
+    c_blk[u] = t * 1024;
+  }
+  auto copy_tile = [&](const half_t* src, char* dst, int tile_idx) __attribute__((always_inline)) {
+    const int row0 = tile_idx * kTile;
+    const half_t* tp = src + (long)row0 * rs;  // wave-uniform
+    if (row0 + kTile <= N) {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) copy16(tp, c_goff[u], dst + c_blk[u]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) {  // rows past the end re-read row N-1
+        const int back = max(row0 + c_row[u] - (N - 1), 0);
+        copy16(tp, c_goff[u] - back * rs * 2, dst + c_blk[u]);
+      }
+    }
+  };
+
+  copy_tile(Kb, k_slot0, 0);
+  if (nt > 1) copy_tile(Kb, k_slot1, 1);
+  copy_tile(Vb, v_slot0, 0);
 
   h8 qf[G::kKSteps];
   {
@@ -290,11 +453,9 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
     }
   }
 
-  int nt = (N + kTile - 1) / kTile;
-  if (CAUSAL) nt = min(nt, (min(m0 + kBlockRes, N) - 1) / kTile + 1);
-
-  const int k_off = lane_rows_off<KS::kRowBytes>(lane);
-  const int v_off = lane_cols_off<VS::kRowBytes>(lane);
+  int k_off[2], v_off[2];
+  swz_rows_off<D>(lane, k_off);
+  swz_cols_off<D>(lane, v_off);
 
   f16v o[G::kDBlocks];
 #pragma unroll
@@ -302,85 +463,109 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
+  f16v s[2];   // scores of the tile in flight
+  h8 pf[4];    // its probabilities, fp16, B-operand order
 
-  KS ks;
-  VS vs;
-  ks.init(rs);
-  vs.init(rs);
-  h8 kreg[KS::kCPT], vreg[VS::kCPT];
-  ks.load(Kb, rs, 0, N, kreg);
-  vs.load(Vb, rs, 0, N, vreg);
-  ks.store(smem, kreg);
-  vs.store(smem + KS::kTileBytes, vreg);
-  __syncthreads();
-
-  for (int kt = 0; kt < nt; ++kt) {
-    const char* Kl = smem + (kt & 1) * kBuf;
-    const char* Vl = Kl + KS::kTileBytes;
-    const bool more = kt + 1 < nt;
-    if (more) {
-      ks.load(Kb, rs, (kt + 1) * kTile, N, kreg);
-      vs.load(Vb, rs, (kt + 1) * kTile, N, vreg);
+  auto scores = [&](const char* Kl, int t) __attribute__((always_inline)) {
+    if (t >= ntw) return;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[rb][r] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(swz_rows<D>(Kl, rb, kk, k_off), qf[kk], s[rb]);
     }
-    const int key0 = kt * kTile;
-    const bool active = !CAUSAL || key0 <= q0w + kResident - 1;
-    if (active) {
-      f16v s[2];
+  };
+  auto softmax = [&](int t) __attribute__((always_inline)) {
+    if (t < 0 || t >= ntw) return;
+    const int key0 = t * kTile;
+    if ((CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N)) {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[rb][r] = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < G::kKSteps; ++kk) {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(lds_rows<KS::kRowBytes>(Kl, rb, kk, k_off), qf[kk], s[rb]);
-      }
-      const bool need_mask = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
-      if (need_mask) {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            int key = key0 + acc_row(rb, r, hh);
-            if ((CAUSAL && key > qi) || key >= N) s[rb][r] = -INFINITY;
-          }
-      }
-      float mx = s[0][0];
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[rb][r]);
-      mx = fmaxf(mx, other_half(mx));
-      const float m_new = fmaxf(m_run, mx);
-      if (__builtin_amdgcn_ballot_w64((m_new - m_run) * c > kRescaleLog2) != 0) {
-        const float alpha = fast_exp2((m_run - m_new) * c);
-        m_run = m_new;
-        l_run *= alpha;
-#pragma unroll
-        for (int db = 0; db < G::kDBlocks; ++db)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
-      }
-      const float mc = m_run * c;
-      h8 pf[4];
-#pragma unroll
-      for (int c16 = 0; c16 < 4; ++c16) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) pf[c16][j] = (half_t)fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + j], c, -mc));
-        l_run = add_halves(pf[c16], l_run);
-      }
-#pragma unroll
-      for (int c16 = 0; c16 < 4; ++c16) {
-#pragma unroll
-        for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(lds_cols<VS::kRowBytes>(Vl, c16, db, v_off), pf[c16], o[db]);
-      }
+        for (int r = 0; r < 16; ++r) {
+          int key = key0 + acc_row(rb, r, hh);
+          if ((CAUSAL && key > qi) || key >= N) s[rb][r] = -INFINITY;
+        }
     }
-    if (more) {
-      char* Kn = smem + ((kt + 1) & 1) * kBuf;
-      ks.store(Kn, kreg);
-      vs.store(Kn + KS::kTileBytes, vreg);
+    float mx = s[0][0];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[rb][r]);
+    mx = fmaxf(mx, other_half(mx));
+    const float m_new = fmaxf(m_run, mx);
+    if (__builtin_amdgcn_ballot_w64((m_new - m_run) * c > kRescaleLog2) != 0) {
+      const float alpha = fast_exp2((m_run - m_new) * c);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
     }
-    __syncthreads();
+    const float mc = m_run * c;
+#pragma unroll
+    for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pf[c16][e] = (half_t)fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + e], c, -mc));
+      l_run = add_halves(pf[c16], l_run);
+    }
+  };
+  auto accumulate = [&](const char* Vl, int t) __attribute__((always_inline)) {
+    if (t < 0 || t >= ntw) return;
+#pragma unroll
+    for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(swz_cols<D>(Vl, c16, db, v_off), pf[c16], o[db]);
+    }
+  };
+
+  const bool first_group = wave < kFwdWaves / 2;
+  // Everything issued so far (Q rows, first copies) is waited for here, once,
+  // so that no wait for a register load is left to be placed inside the loop,
+  // where it would also wait for the copies in flight.
+  wait_vm<0>();
+  // Iteration j with j % 3 == S: K(j) sits in K slot S, V(j-1) in V slot S+2,
+  // K(j+2) is copied into K slot S+2 and V(j+1) into V slot S+1.
+  auto iteration = [&](auto tag, auto group_tag, int j) __attribute__((always_inline)) {
+    constexpr int S = decltype(tag)::value;
+    constexpr bool kFirst = decltype(group_tag)::value == 0;
+    // K(j) and V(j-1) were issued two iterations ago; what the previous
+    // iteration issued (K(j+1), V(j)) may still be in flight.
+    if (j + 1 < nt) wait_vm<2 * kIPW>();
+    else if (j < nt) wait_vm<kIPW>();
+    else wait_vm<0>();
+    block_barrier();
+    if (j + 2 < nt) copy_tile(Kb, k_slot(IntTag<S + 2>{}), j + 2);
+    if (j + 1 < nt) copy_tile(Vb, v_slot(IntTag<S + 1>{}), j + 1);
+    const char* Kl = k_slot(IntTag<S>{});
+    const char* Vl = v_slot(IntTag<S + 2>{});
+    if (kFirst) {
+      accumulate(Vl, j - 1);
+      if (j < nt) { scores(Kl, j); softmax(j); }
+    } else {
+      softmax(j - 1);
+      accumulate(Vl, j - 1);
+      if (j < nt) scores(Kl, j);
+    }
+  };
+  // Each group runs its own copy of the loop: no joins between the two
+  // orders inside the loop, so no register shuffling at branch merges.
+  if (first_group) {
+    for (int j = 0; j <= nt; j += 3) {
+      iteration(IntTag<0>{}, IntTag<0>{}, j);
+      if (j + 1 <= nt) iteration(IntTag<1>{}, IntTag<0>{}, j + 1);
+      if (j + 2 <= nt) iteration(IntTag<2>{}, IntTag<0>{}, j + 2);
+    }
+  } else {
+    for (int j = 0; j <= nt; j += 3) {
+      iteration(IntTag<0>{}, IntTag<1>{}, j);
+      if (j + 1 <= nt) iteration(IntTag<1>{}, IntTag<1>{}, j + 1);
+      if (j + 2 <= nt) iteration(IntTag<2>{}, IntTag<1>{}, j + 2);
+    }
   }
 
   const float l_tot = l_run + other_half(l_run);
@@ -673,12 +858,12 @@ bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) !
 template <int D, bool CAUSAL>
 int launch_forward(const void* q, const void* k, const void* v, void* o, void* lse, int batch, int head, int n,
                    float scale, hipStream_t stream) {
-  const int nmb = (n + kBlockRes - 1) / kBlockRes;
+  const int nmb = (n + kFwdBlockQ - 1) / kFwdBlockQ;
   dim3 grid(nmb * batch * head);
   // scale == 0 would turn the masked scores (-inf) into NaN when multiplied; a
   // tiny positive factor gives the same uniform softmax and keeps -inf * c = -inf.
   const float c = fmaxf(fabsf(scale) * kLog2e, 1e-30f);
-  fmha_fwd_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+  fmha_fwd_kernel<D, CAUSAL><<<grid, kFwdThreads, 0, stream>>>(
       (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, (float*)lse, head, n, nmb, c, scale < 0.f ? 1 : 0);
   return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
 }
