@@ -477,6 +477,15 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(swz_rows<D>(Kl, rb, kk, k_off), qf[kk], s[rb]);
     }
+    // LDS reads run kLead MFMAs ahead of their use.
+    constexpr int kN = 2 * G::kKSteps, kLead = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
+#pragma unroll
+    for (int n = 0; n < kN - kLead; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
   auto softmax = [&](int t) __attribute__((always_inline)) {
     if (t < 0 || t >= ntw) return;
@@ -521,6 +530,15 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 #pragma unroll
       for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(swz_cols<D>(Vl, c16, db, v_off), pf[c16], o[db]);
     }
+    // LDS reads (two per MFMA) run kLead MFMAs ahead of their use.
+    constexpr int kN = 4 * G::kDBlocks, kLead = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead, 0);
+#pragma unroll
+    for (int n = 0; n < kN - kLead; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
 
   const bool first_group = wave < kFwdWaves / 2;
