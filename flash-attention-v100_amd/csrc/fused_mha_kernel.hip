@@ -734,35 +734,115 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 }
 
 // ---------------------------------------------------------------------------
-// Backward, dK/dV pass.  Block = 128 keys, wave = 32 keys, streams Q/dO.
+// Backward, dK/dV pass.  Block = 4 waves = 128 keys, wave = 32 keys, one wave
+// per SIMD (the wave keeps K, V rows and the dK, dV accumulators of its keys in
+// registers); Q/dO tiles of 64 queries stream through a 3-slot LDS ring, copied
+// asynchronously two tiles ahead, together with the tile's lse and delta rows.
 //   S = Q K^T, dP = dO V^T, P = exp(S - lse), dS = P o (dP - delta),
 //   dV^T += dO^T P, dK^T += Q^T dS
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 618-629, 653-656,
 // 697-712; key-block-parallel launch as at :908-915).
 // ---------------------------------------------------------------------------
+constexpr int kKvWaves = 4;
+constexpr int kKvThreads = kKvWaves * 64;
+constexpr int kKvBlockKeys = kKvWaves * kResident;
+
 template <int D, bool CAUSAL>
-__global__ void __launch_bounds__(kThreads, 1)
+__global__ void __launch_bounds__(kKvThreads, 1)
 fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
                      const half_t* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ delta,
-                     half_t* __restrict__ dK, half_t* __restrict__ dV, int H, int N, float c, float scale) {
+                     half_t* __restrict__ dK, half_t* __restrict__ dV, int H, int N, int nnb, float c, float scale) {
   using G = TileGeom<D>;
-  __shared__ __attribute__((aligned(16))) char smem[4 * G::kTileBytes];  // Q0 dO0 Q1 dO1
+  using T = SwzTile<D>;
+  constexpr int kIPW = T::kInstrs / kKvWaves;  // copies per wave per tile, per tensor
+  constexpr int kPerIter = 2 * kIPW + 1;       // Q, dO and one lse/delta copy
+  static_assert(kPerIter < 16, "vmcnt immediate");
+  __shared__ __attribute__((aligned(1024))) char q_slot0[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char q_slot1[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char q_slot2[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char g_slot0[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char g_slot1[T::kBytes];
+  __shared__ __attribute__((aligned(1024))) char g_slot2[T::kBytes];
+  // per wave and slot: 64 lse values then 64 delta values (and 512 bytes unused)
+  __shared__ __attribute__((aligned(1024))) char st_slot0[kKvWaves * 1024];
+  __shared__ __attribute__((aligned(1024))) char st_slot1[kKvWaves * 1024];
+  __shared__ __attribute__((aligned(1024))) char st_slot2[kKvWaves * 1024];
+  auto q_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
+    constexpr int S = decltype(tag)::value % 3;
+    return S == 0 ? q_slot0 : S == 1 ? q_slot1 : q_slot2;
+  };
+  auto g_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
+    constexpr int S = decltype(tag)::value % 3;
+    return S == 0 ? g_slot0 : S == 1 ? g_slot1 : g_slot2;
+  };
+  auto st_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
+    constexpr int S = decltype(tag)::value % 3;
+    return S == 0 ? st_slot0 : S == 1 ? st_slot1 : st_slot2;
+  };
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 31, hh = lane >> 5;
-  const int nblk = blockIdx.x;  // causal: low key blocks are the heavy ones and already come first
-  const int b = blockIdx.y / H, h = blockIdx.y % H;
-  const long rs = (long)H * D;
+  int bh, nblk;
+  slice_and_block(nnb, bh, nblk);  // causal: low key blocks are the heavy ones and come first
+  const int b = bh / H, h = bh - b * H;
+  const int rs = H * D;
   const long head_off = ((long)b * N * H + h) * D;
   const half_t* Qb = Q + head_off;
   const half_t* dOb = dO + head_off;
   const float* lse_b = LSE + ((long)b * H + h) * N;
   const float* delta_b = delta + ((long)b * H + h) * N;
 
-  const int n0 = nblk * kBlockRes;
+  const int n0 = nblk * kKvBlockKeys;
   const int k0w = n0 + wave * kResident;
   const int ki = k0w + i;
   const int krow = min(ki, N - 1);
+
+  const int nt = (N + kTile - 1) / kTile;
+  const int t_begin = CAUSAL ? n0 / kTile : 0;
+  const int n_it = nt - t_begin;  // >= 1
+
+  // this wave's share of every tile copy
+  int c_row[kIPW], c_goff[kIPW], c_blk[kIPW];
+#pragma unroll
+  for (int u = 0; u < kIPW; ++u) {
+    const int t = wave * kIPW + u;
+    copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
+    c_blk[u] = t * 1024;
+  }
+  // lse/delta copy: lanes 0-15 fetch the tile's 64 lse values, lanes 16-31 its
+  // 64 delta values, 4 floats each; lanes 32-63 repeat them into unused space.
+  const int st_quad = (lane & 15) * 4;
+  const bool st_is_delta = (lane >> 4) & 1;
+  auto copy_tiles = [&](char* qdst, char* gdst, char* sdst, int tile_idx) __attribute__((always_inline)) {
+    const int row0 = tile_idx * kTile;
+    const half_t* qp = Qb + (long)row0 * rs;   // wave-uniform
+    const half_t* gp = dOb + (long)row0 * rs;
+    if (row0 + kTile <= N) {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) copy16(qp, c_goff[u], qdst + c_blk[u]);
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) copy16(gp, c_goff[u], gdst + c_blk[u]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) {  // rows past the end re-read row N-1
+        const int back = max(row0 + c_row[u] - (N - 1), 0);
+        copy16(qp, c_goff[u] - back * rs * 2, qdst + c_blk[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) {
+        const int back = max(row0 + c_row[u] - (N - 1), 0);
+        copy16(gp, c_goff[u] - back * rs * 2, gdst + c_blk[u]);
+      }
+    }
+    // N is a multiple of 32, so a quad of rows is either inside or outside [0, N)
+    const int quad = min(row0 + st_quad, N - 4);
+    const float* sp = st_is_delta ? delta_b : lse_b;
+    copy16(reinterpret_cast<const half_t*>(lse_b), (int)((sp - lse_b) + quad) * 4, sdst + wave * 1024);
+  };
+
+  copy_tiles(q_slot0, g_slot0, st_slot0, t_begin);
+  if (n_it > 1) copy_tiles(q_slot1, g_slot1, st_slot1, t_begin + 1);
 
   h8 kf[G::kKSteps], vf[G::kKSteps];
   {
@@ -775,11 +855,10 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     }
   }
 
-  const int nt = (N + kTile - 1) / kTile;
-  const int t_begin = CAUSAL ? n0 / kTile : 0;
-
-  const int lane_row_off = i * G::kRowBytes + hh * 16;
-  const int lane_tr_off = (4 * hh + ((lane & 15) >> 2)) * G::kRowBytes + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  int r_off[2], c_off[2];
+  swz_rows_off<D>(lane, r_off);
+  swz_cols_off<D>(lane, c_off);
+  const int st_off = wave * 1024 + hh * 16;  // + (rb * 32 + 8 * g) * 4: lse quad; + 256: delta quad
 
   f16v dk[G::kDBlocks], dv[G::kDBlocks];
 #pragma unroll
@@ -787,76 +866,71 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
 
-  h8 qreg[G::kChunksPerThread], greg[G::kChunksPerThread];
-  if (t_begin < nt) {
-    tile_load<D>(Qb, rs, t_begin * kTile, N, qreg);
-    tile_load<D>(dOb, rs, t_begin * kTile, N, greg);
-    tile_store<D>(smem, qreg);
-    tile_store<D>(smem + G::kTileBytes, greg);
-  }
-  __syncthreads();
-
-  for (int qt = t_begin; qt < nt; ++qt) {
-    const int buf = (qt - t_begin) & 1;
-    const char* Ql = smem + buf * 2 * G::kTileBytes;
-    const char* Gl = Ql + G::kTileBytes;
-    const bool more = qt + 1 < nt;
-    if (more) {
-      tile_load<D>(Qb, rs, (qt + 1) * kTile, N, qreg);
-      tile_load<D>(dOb, rs, (qt + 1) * kTile, N, greg);
-    }
-    const int q0 = qt * kTile;
-    const bool active = !CAUSAL || q0 + kTile - 1 >= k0w;
-    if (active) {
-      const bool need_mask = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
+  // One 64-query tile.  MASKED tiles straddle the diagonal or the end of the sequence.
+  auto tile = [&](const char* Ql, const char* Gl, const char* Sl, int q0, auto masked_tag) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value != 0;
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-        f16v s, dp;
+    for (int rb = 0; rb < 2; ++rb) {
+      f16v s, dp;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
-        for (int kk = 0; kk < G::kKSteps; ++kk) {
-          s = mfma(read_rows<D>(Ql, rb, kk, lane_row_off), kf[kk], s);
-          dp = mfma(read_rows<D>(Gl, rb, kk, lane_row_off), vf[kk], dp);
-        }
+      for (int kk = 0; kk < G::kKSteps; ++kk) {
+        s = mfma(swz_rows<D>(Ql, rb, kk, r_off), kf[kk], s);
+        dp = mfma(swz_rows<D>(Gl, rb, kk, r_off), vf[kk], dp);
+      }
+      h8 pf[2], dsf[2];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int qg = q0 + rb * 32 + 8 * g + 4 * hh;  // 4 consecutive queries, multiple of 4
-          const int qld = min(qg, N - 4);
-          const f4v l4 = *reinterpret_cast<const f4v*>(lse_b + qld);
-          const f4v d4 = *reinterpret_cast<const f4v*>(delta_b + qld);
+      for (int g = 0; g < 4; ++g) {
+        const f4v l4 = *reinterpret_cast<const f4v*>(Sl + st_off + (rb * 32 + 8 * g) * 4);
+        const f4v d4 = *reinterpret_cast<const f4v*>(Sl + st_off + 256 + (rb * 32 + 8 * g) * 4);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = 4 * g + e;
-            float p = fast_exp2(fmaf(s[r], c, -l4[e] * kLog2e));
-            if (need_mask) {
-              int q = qg + e;
-              if ((CAUSAL && ki > q) || q >= N) p = 0.f;
-            }
-            s[r] = p;
-            dp[r] = p * (dp[r] - d4[e]);
+        for (int e = 0; e < 4; ++e) {
+          const int r = 4 * g + e;
+          float p = fast_exp2(fmaf(s[r], c, -l4[e] * kLog2e));
+          if (MASKED) {
+            const int q = q0 + rb * 32 + 8 * g + 4 * hh + e;
+            if ((CAUSAL && ki > q) || q >= N) p = 0.f;
           }
+          const float ds = p * (dp[r] - d4[e]);
+          pf[g >> 1][(g & 1) * 4 + e] = (half_t)p;
+          dsf[g >> 1][(g & 1) * 4 + e] = (half_t)ds;
         }
+      }
 #pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-          const h8 pf = pack8(s, cc * 8);
-          const h8 dsf = pack8(dp, cc * 8);
-          const int c16 = rb * 2 + cc;
+      for (int cc = 0; cc < 2; ++cc) {
+        const int c16 = rb * 2 + cc;
 #pragma unroll
-          for (int db = 0; db < G::kDBlocks; ++db) {
-            dv[db] = mfma(read_cols<D>(Gl, c16, db, lane_tr_off), pf, dv[db]);
-            dk[db] = mfma(read_cols<D>(Ql, c16, db, lane_tr_off), dsf, dk[db]);
-          }
+        for (int db = 0; db < G::kDBlocks; ++db) {
+          dv[db] = mfma(swz_cols<D>(Gl, c16, db, c_off), pf[cc], dv[db]);
+          dk[db] = mfma(swz_cols<D>(Ql, c16, db, c_off), dsf[cc], dk[db]);
         }
       }
     }
-    if (more) {
-      char* Qn = smem + (buf ^ 1) * 2 * G::kTileBytes;
-      tile_store<D>(Qn, qreg);
-      tile_store<D>(Qn + G::kTileBytes, greg);
+  };
+
+  wait_vm<0>();  // K/V rows and the first copies: nothing is left for the compiler to wait on in the loop
+  auto iteration = [&](auto tag, int it) __attribute__((always_inline)) {
+    constexpr int S = decltype(tag)::value;
+    // tile `it` was issued two iterations ago; the copies of tile it+1 may still be in flight
+    if (it + 1 < n_it) wait_vm<kPerIter>();
+    else wait_vm<0>();
+    block_barrier();
+    if (it + 2 < n_it) copy_tiles(q_slot(IntTag<S + 2>{}), g_slot(IntTag<S + 2>{}), st_slot(IntTag<S + 2>{}), t_begin + it + 2);
+    const int q0 = (t_begin + it) * kTile;
+    const bool active = !CAUSAL || q0 + kTile - 1 >= k0w;
+    if (active) {
+      const bool masked = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
+      if (masked) tile(q_slot(IntTag<S>{}), g_slot(IntTag<S>{}), st_slot(IntTag<S>{}), q0, IntTag<1>{});
+      else tile(q_slot(IntTag<S>{}), g_slot(IntTag<S>{}), st_slot(IntTag<S>{}), q0, IntTag<0>{});
     }
-    __syncthreads();
+  };
+  for (int it = 0; it < n_it; it += 3) {
+    iteration(IntTag<0>{}, it);
+    if (it + 1 < n_it) iteration(IntTag<1>{}, it + 1);
+    if (it + 2 < n_it) iteration(IntTag<2>{}, it + 2);
   }
+
   store_resident<D>(dK + head_off, rs, ki, N, dk, scale, hh);
   store_resident<D>(dV + head_off, rs, ki, N, dv, 1.f, hh);
 }
@@ -908,9 +982,10 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   if (passes & kPassDkDv) {
-    fmha_bwd_dkdv_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+    const int nnb = (n + kKvBlockKeys - 1) / kKvBlockKeys;
+    fmha_bwd_dkdv_kernel<D, CAUSAL><<<dim3(nnb * batch * head), kKvThreads, 0, stream>>>(
         (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
-        (half_t*)dk, (half_t*)dv, head, n, c, scale);
+        (half_t*)dk, (half_t*)dv, head, n, nnb, c, scale);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   return FUSED_MHA_OK;
