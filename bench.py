@@ -104,7 +104,7 @@ def kernel_times(B, H, N, D, causal, steps, warmup):
     c = int(causal)
     calls = {
         "fmha_fwd_kernel": lambda: lib.fused_mha_forward(p(q), p(k), p(v), p(out), p(lse), B, H, N, N, D, scale, c, s),
-        "fmha_bwd_delta_kernel": lambda: lib.fused_mha_backward_delta(p(out), p(do), p(ws), nbytes, B, H, N, D, s),
+        "fmha_bwd_delta_kernel": lambda: lib.fused_mha_backward_delta(p(out), p(do), p(lse), p(ws), nbytes, B, H, N, D, s),
         "fmha_bwd_dq_kernel": lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dq),
                                                                  B, H, N, D, scale, c, s),
         "fmha_bwd_dkdv_kernel": lambda: lib.fused_mha_backward_dkdv(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes,

@@ -371,24 +371,11 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kFwdWaves;  // copy instructions per wave per tile
-  // Ring slots are separate arrays, indexed with compile-time constants only, so
-  // the compiler can tell which slot an asynchronous copy writes and does not
-  // make LDS reads of the other slots wait for copies still in flight.
-  static_assert(kRing == 3, "the main loop is unrolled for three slots");
-  __shared__ __attribute__((aligned(1024))) char k_slot0[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char k_slot1[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char k_slot2[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char v_slot0[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char v_slot1[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char v_slot2[T::kBytes];
-  auto k_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
-    constexpr int S = decltype(tag)::value % kRing;
-    return S == 0 ? k_slot0 : S == 1 ? k_slot1 : k_slot2;
-  };
-  auto v_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
-    constexpr int S = decltype(tag)::value % kRing;
-    return S == 0 ? v_slot0 : S == 1 ? v_slot1 : v_slot2;
-  };
+  // K ring then V ring, kRing slots each.  The copies into the ring are inline
+  // asm (see copy16), so slots can be addressed at run time.
+  __shared__ __attribute__((aligned(1024))) char smem[2 * kRing * T::kBytes];
+  char* const k_ring = smem;
+  char* const v_ring = smem + kRing * T::kBytes;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -439,9 +426,9 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
     }
   };
 
-  copy_tile(Kb, k_slot0, 0);
-  if (nt > 1) copy_tile(Kb, k_slot1, 1);
-  copy_tile(Vb, v_slot0, 0);
+  copy_tile(Kb, k_ring, 0);
+  if (nt > 1) copy_tile(Kb, k_ring + T::kBytes, 1);
+  copy_tile(Vb, v_ring, 0);
 
   h8 qf[G::kKSteps];
   {
@@ -546,45 +533,37 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   // so that no wait for a register load is left to be placed inside the loop,
   // where it would also wait for the copies in flight.
   wait_vm<0>();
-  // Iteration j with j % 3 == S: K(j) sits in K slot S, V(j-1) in V slot S+2,
-  // K(j+2) is copied into K slot S+2 and V(j+1) into V slot S+1.
-  auto iteration = [&](auto tag, auto group_tag, int j) __attribute__((always_inline)) {
-    constexpr int S = decltype(tag)::value;
+  // Iteration j: K(j) sits in K slot j % 3, V(j-1) in V slot (j-1) % 3; K(j+2)
+  // is copied into K slot (j+2) % 3 and V(j+1) into V slot (j+1) % 3.
+  auto run = [&](auto group_tag) __attribute__((always_inline)) {
     constexpr bool kFirst = decltype(group_tag)::value == 0;
-    // K(j) and V(j-1) were issued two iterations ago; what the previous
-    // iteration issued (K(j+1), V(j)) may still be in flight.
-    if (j + 1 < nt) wait_vm<2 * kIPW>();
-    else if (j < nt) wait_vm<kIPW>();
-    else wait_vm<0>();
-    block_barrier();
-    if (j + 2 < nt) copy_tile(Kb, k_slot(IntTag<S + 2>{}), j + 2);
-    if (j + 1 < nt) copy_tile(Vb, v_slot(IntTag<S + 1>{}), j + 1);
-    const char* Kl = k_slot(IntTag<S>{});
-    const char* Vl = v_slot(IntTag<S + 2>{});
-    if (kFirst) {
-      accumulate(Vl, j - 1);
-      if (j < nt) { scores(Kl, j); softmax(j); }
-    } else {
-      softmax(j - 1);
-      accumulate(Vl, j - 1);
-      if (j < nt) scores(Kl, j);
+    int s0 = 0, s1 = 1, s2 = 2;  // j % 3, (j+1) % 3, (j+2) % 3
+    for (int j = 0; j <= nt; ++j) {
+      // K(j) and V(j-1) were issued two iterations ago; what the previous
+      // iteration issued (K(j+1), V(j)) may still be in flight.
+      if (j + 1 < nt) wait_vm<2 * kIPW>();
+      else if (j < nt) wait_vm<kIPW>();
+      else wait_vm<0>();
+      block_barrier();
+      if (j + 2 < nt) copy_tile(Kb, k_ring + s2 * T::kBytes, j + 2);
+      if (j + 1 < nt) copy_tile(Vb, v_ring + s1 * T::kBytes, j + 1);
+      const char* Kl = k_ring + s0 * T::kBytes;
+      const char* Vl = v_ring + s2 * T::kBytes;
+      if (kFirst) {
+        accumulate(Vl, j - 1);
+        if (j < nt) { scores(Kl, j); softmax(j); }
+      } else {
+        softmax(j - 1);
+        accumulate(Vl, j - 1);
+        if (j < nt) scores(Kl, j);
+      }
+      const int t = s0; s0 = s1; s1 = s2; s2 = t;
     }
   };
   // Each group runs its own copy of the loop: no joins between the two
   // orders inside the loop, so no register shuffling at branch merges.
-  if (first_group) {
-    for (int j = 0; j <= nt; j += 3) {
-      iteration(IntTag<0>{}, IntTag<0>{}, j);
-      if (j + 1 <= nt) iteration(IntTag<1>{}, IntTag<0>{}, j + 1);
-      if (j + 2 <= nt) iteration(IntTag<2>{}, IntTag<0>{}, j + 2);
-    }
-  } else {
-    for (int j = 0; j <= nt; j += 3) {
-      iteration(IntTag<0>{}, IntTag<1>{}, j);
-      if (j + 1 <= nt) iteration(IntTag<1>{}, IntTag<1>{}, j + 1);
-      if (j + 2 <= nt) iteration(IntTag<2>{}, IntTag<1>{}, j + 2);
-    }
-  }
+  if (first_group) run(IntTag<0>{});
+  else run(IntTag<1>{});
 
   const float l_tot = l_run + other_half(l_run);
   const float inv = 1.f / l_tot;
@@ -595,12 +574,14 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 // ---------------------------------------------------------------------------
 // delta[b][h][n] = sum_d dO * O in fp32.  One 16-byte chunk per thread.
 // Takes the place of the two PyTorch ops at reference
-// flash_attn_interface.py:43-44 (which work in fp16).
+// flash_attn_interface.py:43-44 (which work in fp16).  Also writes the
+// logsumexp scaled to the exp2 domain, lse2 = lse * log2(e), behind delta in
+// the workspace, so the dK/dV pass gets both row statistics with one copy.
 // ---------------------------------------------------------------------------
 template <int D>
 __global__ void __launch_bounds__(256)
-fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ dO, float* __restrict__ delta,
-                      int H, int N, long rows) {
+fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ dO, const float* __restrict__ LSE,
+                      float* __restrict__ delta, float* __restrict__ lse2, int H, int N, long rows) {
   constexpr int kLanesPerRow = D / 8;
   const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const long row = t / kLanesPerRow;  // (b*N + n)*H + h
@@ -619,7 +600,9 @@ fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ d
     const int h = (int)(row % H);
     const long b = bn / N;
     const int n = (int)(bn % N);
-    delta[(b * H + h) * N + n] = acc;
+    const long at = (b * H + h) * N + n;
+    delta[at] = acc;
+    lse2[at] = LSE[at] * kLog2e;
   }
 }
 
@@ -743,6 +726,9 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 618-629, 653-656,
 // 697-712; key-block-parallel launch as at :908-915).
 // ---------------------------------------------------------------------------
+#ifndef KV_HINTS
+#define KV_HINTS 1
+#endif
 constexpr int kKvWaves = 4;
 constexpr int kKvThreads = kKvWaves * 64;
 constexpr int kKvBlockKeys = kKvWaves * kResident;
@@ -750,35 +736,21 @@ constexpr int kKvBlockKeys = kKvWaves * kResident;
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(kKvThreads, 1)
 fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-                     const half_t* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ delta,
+                     const half_t* __restrict__ dO, const float* __restrict__ delta, const float* __restrict__ lse2,
                      half_t* __restrict__ dK, half_t* __restrict__ dV, int H, int N, int nnb, float c, float scale) {
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kKvWaves;  // copies per wave per tile, per tensor
   constexpr int kPerIter = 2 * kIPW + 1;       // Q, dO and one lse/delta copy
   static_assert(kPerIter < 16, "vmcnt immediate");
-  __shared__ __attribute__((aligned(1024))) char q_slot0[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char q_slot1[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char q_slot2[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char g_slot0[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char g_slot1[T::kBytes];
-  __shared__ __attribute__((aligned(1024))) char g_slot2[T::kBytes];
-  // per wave and slot: 64 lse values then 64 delta values (and 512 bytes unused)
-  __shared__ __attribute__((aligned(1024))) char st_slot0[kKvWaves * 1024];
-  __shared__ __attribute__((aligned(1024))) char st_slot1[kKvWaves * 1024];
-  __shared__ __attribute__((aligned(1024))) char st_slot2[kKvWaves * 1024];
-  auto q_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
-    constexpr int S = decltype(tag)::value % 3;
-    return S == 0 ? q_slot0 : S == 1 ? q_slot1 : q_slot2;
-  };
-  auto g_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
-    constexpr int S = decltype(tag)::value % 3;
-    return S == 0 ? g_slot0 : S == 1 ? g_slot1 : g_slot2;
-  };
-  auto st_slot = [&](auto tag) __attribute__((always_inline)) -> char* {
-    constexpr int S = decltype(tag)::value % 3;
-    return S == 0 ? st_slot0 : S == 1 ? st_slot1 : st_slot2;
-  };
+  // Q ring, dO ring, then per slot and wave 64 lse2 values followed by 64 delta
+  // values (and 512 bytes unused).  Slots are addressed at run time; the copies
+  // into them are inline asm (see copy16).
+  __shared__ __attribute__((aligned(1024))) char smem[3 * (2 * T::kBytes + kKvWaves * 1024)];
+  char* const q_ring = smem;
+  char* const g_ring = smem + 3 * T::kBytes;
+  char* const st_ring = smem + 6 * T::kBytes;
+  constexpr int kStBytes = kKvWaves * 1024;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -790,8 +762,8 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   const long head_off = ((long)b * N * H + h) * D;
   const half_t* Qb = Q + head_off;
   const half_t* dOb = dO + head_off;
-  const float* lse_b = LSE + ((long)b * H + h) * N;
   const float* delta_b = delta + ((long)b * H + h) * N;
+  const int lse2_off = (int)(lse2 - delta) * 4;  // bytes from the delta row to the lse2 row; lse2 lies behind delta
 
   const int n0 = nblk * kKvBlockKeys;
   const int k0w = n0 + wave * kResident;
@@ -837,12 +809,11 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     }
     // N is a multiple of 32, so a quad of rows is either inside or outside [0, N)
     const int quad = min(row0 + st_quad, N - 4);
-    const float* sp = st_is_delta ? delta_b : lse_b;
-    copy16(reinterpret_cast<const half_t*>(lse_b), (int)((sp - lse_b) + quad) * 4, sdst + wave * 1024);
+    copy16(reinterpret_cast<const half_t*>(delta_b), quad * 4 + (st_is_delta ? 0 : lse2_off), sdst + wave * 1024);
   };
 
-  copy_tiles(q_slot0, g_slot0, st_slot0, t_begin);
-  if (n_it > 1) copy_tiles(q_slot1, g_slot1, st_slot1, t_begin + 1);
+  copy_tiles(q_ring, g_ring, st_ring, t_begin);
+  if (n_it > 1) copy_tiles(q_ring + T::kBytes, g_ring + T::kBytes, st_ring + kStBytes, t_begin + 1);
 
   h8 kf[G::kKSteps], vf[G::kKSteps];
   {
@@ -867,19 +838,24 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
 
   // One 64-query tile.  MASKED tiles straddle the diagonal or the end of the sequence.
+  // Written as four MFMA stretches (scores of both 32-query halves, then the two
+  // gradient updates) with the element-wise work of a half placed next to an MFMA
+  // stretch that does not depend on it, all in one basic block, so the scheduler
+  // can run VALU work in the shadow of MFMAs.
   auto tile = [&](const char* Ql, const char* Gl, const char* Sl, int q0, auto masked_tag) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value != 0;
+    f16v s[2], dp[2];
+    h8 pf[2][2], dsf[2][2];
+    auto gemm1 = [&](int rb) __attribute__((always_inline)) {
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
-      f16v s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int r = 0; r < 16; ++r) { s[rb][r] = 0.f; dp[rb][r] = 0.f; }
 #pragma unroll
       for (int kk = 0; kk < G::kKSteps; ++kk) {
-        s = mfma(swz_rows<D>(Ql, rb, kk, r_off), kf[kk], s);
-        dp = mfma(swz_rows<D>(Gl, rb, kk, r_off), vf[kk], dp);
+        s[rb] = mfma(swz_rows<D>(Ql, rb, kk, r_off), kf[kk], s[rb]);
+        dp[rb] = mfma(swz_rows<D>(Gl, rb, kk, r_off), vf[kk], dp[rb]);
       }
-      h8 pf[2], dsf[2];
+    };
+    auto pointwise = [&](int rb) __attribute__((always_inline)) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const f4v l4 = *reinterpret_cast<const f4v*>(Sl + st_off + (rb * 32 + 8 * g) * 4);
@@ -887,48 +863,101 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * g + e;
-          float p = fast_exp2(fmaf(s[r], c, -l4[e] * kLog2e));
+          float p = fast_exp2(fmaf(s[rb][r], c, -l4[e]));
           if (MASKED) {
             const int q = q0 + rb * 32 + 8 * g + 4 * hh + e;
             if ((CAUSAL && ki > q) || q >= N) p = 0.f;
           }
-          const float ds = p * (dp[r] - d4[e]);
-          pf[g >> 1][(g & 1) * 4 + e] = (half_t)p;
-          dsf[g >> 1][(g & 1) * 4 + e] = (half_t)ds;
+          const float ds = p * (dp[rb][r] - d4[e]);
+          pf[rb][g >> 1][(g & 1) * 4 + e] = (half_t)p;
+          dsf[rb][g >> 1][(g & 1) * 4 + e] = (half_t)ds;
         }
       }
+    };
+    auto gemm2 = [&](int rb) __attribute__((always_inline)) {
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
         const int c16 = rb * 2 + cc;
 #pragma unroll
         for (int db = 0; db < G::kDBlocks; ++db) {
-          dv[db] = mfma(swz_cols<D>(Gl, c16, db, c_off), pf[cc], dv[db]);
-          dk[db] = mfma(swz_cols<D>(Ql, c16, db, c_off), dsf[cc], dk[db]);
+          dv[db] = mfma(swz_cols<D>(Gl, c16, db, c_off), pf[rb][cc], dv[db]);
+          dk[db] = mfma(swz_cols<D>(Ql, c16, db, c_off), dsf[rb][cc], dk[db]);
         }
       }
+    };
+    gemm1(0);
+    gemm1(1);
+    pointwise(0);
+    gemm2(0);
+    pointwise(1);
+    gemm2(1);
+#if KV_HINTS == 2
+    // Order for the scheduler (masks: 0x008 MFMA, 0x100 LDS read, 0x002 VALU):
+    // LDS reads run ahead of the MFMAs that use them, and the element-wise work of
+    // half 0 / half 1 is spread over the MFMAs of gemm1(1) / gemm2(0).
+    constexpr int kM = 2 * G::kKSteps;  // MFMAs per gemm1 half == per gemm2 half
+    constexpr int kLead = 4;
+    constexpr int kValuPerMfma = 7;
+    __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
+#pragma unroll
+    for (int n = 0; n < kM; ++n) {  // gemm1(0); its reads continue into gemm1(1)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // lse / delta of half 0
+#pragma unroll
+    for (int n = 0; n < kM; ++n) {  // gemm1(1) with pointwise(0)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (n < kM - kLead) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead + 8, 0);  // first gemm2 operands, lse / delta of half 1
+#pragma unroll
+    for (int n = 0; n < kM; ++n) {  // gemm2(0) with pointwise(1)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
+    }
+#pragma unroll
+    for (int n = 0; n < kM; ++n) {  // gemm2(1)
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (n < kM - kLead) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+#elif KV_HINTS == 1
+    // LDS reads run kLead MFMAs ahead of their use inside each MFMA stretch.
+    constexpr int kM1 = 4 * G::kKSteps, kM2 = 4 * G::kKSteps, kLead1 = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, kLead1, 0);
+#pragma unroll
+    for (int n = 0; n < kM1 - kLead1; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead1, 0);
+    (void)kM2;
+#endif
   };
 
   wait_vm<0>();  // K/V rows and the first copies: nothing is left for the compiler to wait on in the loop
-  auto iteration = [&](auto tag, int it) __attribute__((always_inline)) {
-    constexpr int S = decltype(tag)::value;
+  int s0 = 0, s2 = 2;  // it % 3, (it + 2) % 3
+  for (int it = 0; it < n_it; ++it) {
     // tile `it` was issued two iterations ago; the copies of tile it+1 may still be in flight
     if (it + 1 < n_it) wait_vm<kPerIter>();
     else wait_vm<0>();
     block_barrier();
-    if (it + 2 < n_it) copy_tiles(q_slot(IntTag<S + 2>{}), g_slot(IntTag<S + 2>{}), st_slot(IntTag<S + 2>{}), t_begin + it + 2);
+    if (it + 2 < n_it)
+      copy_tiles(q_ring + s2 * T::kBytes, g_ring + s2 * T::kBytes, st_ring + s2 * kStBytes, t_begin + it + 2);
+    const char* Ql = q_ring + s0 * T::kBytes;
+    const char* Gl = g_ring + s0 * T::kBytes;
+    const char* Sl = st_ring + s0 * kStBytes;
     const int q0 = (t_begin + it) * kTile;
     const bool active = !CAUSAL || q0 + kTile - 1 >= k0w;
     if (active) {
       const bool masked = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
-      if (masked) tile(q_slot(IntTag<S>{}), g_slot(IntTag<S>{}), st_slot(IntTag<S>{}), q0, IntTag<1>{});
-      else tile(q_slot(IntTag<S>{}), g_slot(IntTag<S>{}), st_slot(IntTag<S>{}), q0, IntTag<0>{});
+      if (masked) tile(Ql, Gl, Sl, q0, IntTag<1>{});
+      else tile(Ql, Gl, Sl, q0, IntTag<0>{});
     }
-  };
-  for (int it = 0; it < n_it; it += 3) {
-    iteration(IntTag<0>{}, it);
-    if (it + 1 < n_it) iteration(IntTag<1>{}, it + 1);
-    if (it + 2 < n_it) iteration(IntTag<2>{}, it + 2);
+    s2 = s0;
+    s0 = s0 == 2 ? 0 : s0 + 1;
   }
 
   store_resident<D>(dK + head_off, rs, ki, N, dk, scale, hh);
@@ -970,7 +999,7 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
     const long rows = (long)batch * n * head;
     const long threads = rows * (D / 8);
     fmha_bwd_delta_kernel<D><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(
-        (const half_t*)o, (const half_t*)d_o, delta, head, n, rows);
+        (const half_t*)o, (const half_t*)d_o, (const float*)lse, delta, delta + (long)batch * head * n, head, n, rows);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
@@ -984,7 +1013,7 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
   if (passes & kPassDkDv) {
     const int nnb = (n + kKvBlockKeys - 1) / kKvBlockKeys;
     fmha_bwd_dkdv_kernel<D, CAUSAL><<<dim3(nnb * batch * head), kKvThreads, 0, stream>>>(
-        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
+        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, delta, delta + (long)batch * head * n,
         (half_t*)dk, (half_t*)dv, head, n, nnb, c, scale);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
@@ -995,12 +1024,12 @@ int dispatch_backward(int passes, const void* q, const void* k, const void* v, c
                       const void* lse, void* workspace, size_t workspace_bytes, void* dq, void* dk, void* dv,
                       int batch, int head, int m, int n, int d, float scale, int causal, void* stream) {
   const bool need_o = passes & kPassDelta, need_dq = passes & kPassDq, need_dkdv = passes & kPassDkDv;
-  if (!d_o || !workspace || (need_o && !o) || ((need_dq || need_dkdv) && (!q || !k || !v || !lse)) ||
+  if (!d_o || !workspace || !lse || (need_o && !o) || ((need_dq || need_dkdv) && (!q || !k || !v)) ||
       (need_dq && !dq) || (need_dkdv && (!dk || !dv)))
     return FUSED_MHA_ERR_NULL_POINTER;
   if (int rc = check_shape(batch, head, m, n, d)) return rc;
   if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
-  if (workspace_bytes < (size_t)batch * head * n * sizeof(float)) return FUSED_MHA_ERR_BAD_SHAPE;
+  if (workspace_bytes < 2 * (size_t)batch * head * n * sizeof(float)) return FUSED_MHA_ERR_BAD_SHAPE;
   if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(o) || misaligned(d_o) || misaligned(lse) ||
       misaligned(workspace) || misaligned(dq) || misaligned(dk) || misaligned(dv))
     return FUSED_MHA_ERR_MISALIGNED;
@@ -1037,7 +1066,7 @@ int fused_mha_forward(const void* query_ptr, const void* key_ptr, const void* va
 
 size_t fused_mha_backward_workspace_bytes(int batch, int head, int n, int d) {
   if (check_shape(batch, head, n, n, d) != FUSED_MHA_OK) return 0;
-  return (size_t)batch * head * n * sizeof(float);
+  return 2 * (size_t)batch * head * n * sizeof(float);  // delta and lse * log2(e), fp32 (batch, head, n) each
 }
 
 int fused_mha_backward(const void* query_ptr, const void* key_ptr, const void* value_ptr, const void* output_ptr,
@@ -1049,9 +1078,9 @@ int fused_mha_backward(const void* query_ptr, const void* key_ptr, const void* v
                            stream);
 }
 
-int fused_mha_backward_delta(const void* output_ptr, const void* d_output_ptr, void* workspace,
+int fused_mha_backward_delta(const void* output_ptr, const void* d_output_ptr, const void* lse_ptr, void* workspace,
                              size_t workspace_bytes, int batch, int head, int n, int d, void* stream) {
-  return dispatch_backward(kPassDelta, nullptr, nullptr, nullptr, output_ptr, d_output_ptr, nullptr, workspace,
+  return dispatch_backward(kPassDelta, nullptr, nullptr, nullptr, output_ptr, d_output_ptr, lse_ptr, workspace,
                            workspace_bytes, nullptr, nullptr, nullptr, batch, head, n, n, d, 1.f, 0, stream);
 }
 

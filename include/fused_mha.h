@@ -54,7 +54,8 @@ int fused_mha_forward(const void *query_ptr, const void *key_ptr, const void *va
 
 /*
  * Bytes of device scratch fused_mha_backward needs for this problem size
- * (holds delta = rowsum(d_o * o) in fp32, shape (batch, head, n)).
+ * (holds delta = rowsum(d_o * o) and lse * log2(e), both fp32 of shape
+ * (batch, head, n), delta first).
  * Returns 0 for an invalid shape.  No counterpart in the reference, which
  * receives delta from Python (flash_attn_interface.py:43-44).
  */
@@ -82,11 +83,12 @@ int fused_mha_backward(const void *query_ptr, const void *key_ptr, const void *v
  * streams.  Same conventions and workspace as fused_mha_backward.  No
  * counterpart in the reference, whose backward is a single kernel
  * (kernel/fused_mha_kernel.cu:904-916).
- *   delta : workspace[b][h][i] = sum_j d_o[b][i][h][j] * o[b][i][h][j]  (fp32)
+ *   delta : workspace[b][h][i] = sum_j d_o[b][i][h][j] * o[b][i][h][j]  (fp32),
+ *           followed by lse * log2(e) in the same shape
  *   dq    : d_q, streaming key/value tiles per block of 128 queries
  *   dkdv  : d_k and d_v, streaming query/d_o tiles per block of 128 keys
  */
-int fused_mha_backward_delta(const void *output_ptr, const void *d_output_ptr,
+int fused_mha_backward_delta(const void *output_ptr, const void *d_output_ptr, const void *lse_ptr,
                              void *workspace, size_t workspace_bytes,
                              int batch, int head, int n, int d, void *stream);
 int fused_mha_backward_dq(const void *query_ptr, const void *key_ptr, const void *value_ptr,

@@ -37,7 +37,7 @@ def load():
     lib.fused_mha_backward_workspace_bytes.restype = _sz
     lib.fused_mha_backward.argtypes = [_vp] * 7 + [_sz] + [_vp] * 3 + [_i] * 5 + [_f, _i, _vp]
     lib.fused_mha_backward.restype = _i
-    lib.fused_mha_backward_delta.argtypes = [_vp, _vp, _vp, _sz] + [_i] * 4 + [_vp]
+    lib.fused_mha_backward_delta.argtypes = [_vp, _vp, _vp, _vp, _sz] + [_i] * 4 + [_vp]
     lib.fused_mha_backward_delta.restype = _i
     lib.fused_mha_backward_dq.argtypes = [_vp] * 6 + [_sz, _vp] + [_i] * 4 + [_f, _i, _vp]
     lib.fused_mha_backward_dq.restype = _i
@@ -67,7 +67,7 @@ def backward(lib, q, k, v, out, dout, lse, scale, causal, stream=None, split=Fal
     dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream
     if split:
-        rc = lib.fused_mha_backward_delta(out.data_ptr(), dout.data_ptr(), ws.data_ptr(), nbytes, B, H, N, D, s)
+        rc = lib.fused_mha_backward_delta(out.data_ptr(), dout.data_ptr(), lse.data_ptr(), ws.data_ptr(), nbytes, B, H, N, D, s)
         assert rc == OK, lib.fused_mha_error_string(rc)
         rc = lib.fused_mha_backward_dkdv(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
                                          ws.data_ptr(), nbytes, dk.data_ptr(), dv.data_ptr(), B, H, N, D, scale,
@@ -80,4 +80,4 @@ def backward(lib, q, k, v, out, dout, lse, scale, causal, stream=None, split=Fal
                                     lse.data_ptr(), ws.data_ptr(), nbytes, dq.data_ptr(), dk.data_ptr(),
                                     dv.data_ptr(), B, H, N, N, D, scale, int(causal), s)
     assert rc == OK, lib.fused_mha_error_string(rc)
-    return dq, dk, dv, ws.view(torch.float32).view(B, H, N)
+    return dq, dk, dv, ws.view(torch.float32)[:B * H * N].view(B, H, N)

@@ -35,8 +35,8 @@ def test_error_strings(lib):
 
 
 def test_workspace_bytes(lib):
-    assert lib.fused_mha_backward_workspace_bytes(2, 32, 4096, 128) == 2 * 32 * 4096 * 4
-    assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 64) == 4 * 128 * 4
+    assert lib.fused_mha_backward_workspace_bytes(2, 32, 4096, 128) == 2 * 2 * 32 * 4096 * 4
+    assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 64) == 2 * 4 * 128 * 4
     assert lib.fused_mha_backward_workspace_bytes(1, 4, 100, 64) == 0
     assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 96) == 0
 
@@ -59,14 +59,14 @@ def test_forward_validation_codes(lib):
 def test_backward_validation_codes(lib):
     p = 0x1000
     b = lib.fused_mha_backward
-    ws = 1 * 1 * 32 * 4
+    ws = 2 * 1 * 1 * 32 * 4
     assert b(p, p, p, p, p, p, None, ws, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
     assert b(p, p, p, p, p, p, p, ws, p, p, None, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
     assert b(p, p, p, p, p, p, p, ws - 1, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE
     assert b(p, p, p, p, p, p, p, ws, p, p, p, 1, 1, 40, 40, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE
     assert b(p, p, p, p, p, p, p, ws, p, p, p, 1, 1, 32, 32, 32, 1.0, 0, None) == abi.ERR_BAD_HEAD_DIM
     assert b(p, p, p, p, p, p, p, ws, p, p + 8, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_MISALIGNED
-    assert lib.fused_mha_backward_delta(p, None, p, ws, 1, 1, 32, 64, None) == abi.ERR_NULL_POINTER
+    assert lib.fused_mha_backward_delta(p, None, p, p, ws, 1, 1, 32, 64, None) == abi.ERR_NULL_POINTER
     assert lib.fused_mha_backward_dq(p, p, p, p, p, p, ws, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
     assert lib.fused_mha_backward_dkdv(p, p, p, p, p, p, ws, p, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
 
