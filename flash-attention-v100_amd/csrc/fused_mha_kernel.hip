@@ -607,31 +607,85 @@ fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ d
 }
 
 // ---------------------------------------------------------------------------
-// Backward, dQ pass.  Block = 128 queries, wave = 32 queries, streams K/V.
+// Backward, dQ pass.  Block = 8 waves = 256 queries, wave = 32 queries; K/V
+// tiles of 64 keys stream through a 3-slot LDS ring, copied two tiles ahead.
 //   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T o (dP^T - delta), dQ^T += K^T dS^T
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 653-656, 680-683).
+// lse and delta belong to the resident query, so they are per-lane scalars.
 // ---------------------------------------------------------------------------
+constexpr int kDqWaves = 4;
+constexpr int kDqThreads = kDqWaves * 64;
+constexpr int kDqBlockQ = kDqWaves * kResident;
+
 template <int D, bool CAUSAL>
-__global__ void __launch_bounds__(kThreads, 2)
+__global__ void __launch_bounds__(kDqThreads, 1)
 fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
                    const half_t* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ delta,
-                   half_t* __restrict__ dQ, int H, int N, float c, float scale) {
+                   half_t* __restrict__ dQ, int H, int N, int nmb, float c, float scale) {
   using G = TileGeom<D>;
-  __shared__ __attribute__((aligned(16))) char smem[4 * G::kTileBytes];  // K0 V0 K1 V1
+  using T = SwzTile<D>;
+  constexpr int kIPW = T::kInstrs / kDqWaves;  // copies per wave per tile, per tensor
+  __shared__ __attribute__((aligned(1024))) char smem[2 * 3 * T::kBytes];  // K ring, V ring
+  char* const k_ring = smem;
+  char* const v_ring = smem + 3 * T::kBytes;
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 31, hh = lane >> 5;
-  const int mblk = CAUSAL ? (int)(gridDim.x - 1 - blockIdx.x) : (int)blockIdx.x;
-  const int b = blockIdx.y / H, h = blockIdx.y % H;
-  const long rs = (long)H * D;
+  int bh, mb;
+  slice_and_block(nmb, bh, mb);
+  const int mblk = CAUSAL ? nmb - 1 - mb : mb;  // heavy blocks first
+  const int b = bh / H, h = bh - b * H;
+  const int rs = H * D;
   const long head_off = ((long)b * N * H + h) * D;
   const half_t* Kb = K + head_off;
   const half_t* Vb = V + head_off;
 
-  const int m0 = mblk * kBlockRes;
+  const int m0 = mblk * kDqBlockQ;
   const int q0w = m0 + wave * kResident;
   const int qi = q0w + i;
   const int qrow = min(qi, N - 1);
+
+  int nt = (N + kTile - 1) / kTile;
+  int ntw = nt;
+  if (CAUSAL) {
+    nt = min(nt, (min(m0 + kDqBlockQ, N) - 1) / kTile + 1);
+    ntw = min(nt, (min(q0w + kResident, N) - 1) / kTile + 1);
+    if (q0w >= N) ntw = 0;
+  }
+
+  int c_row[kIPW], c_goff[kIPW], c_blk[kIPW];
+#pragma unroll
+  for (int u = 0; u < kIPW; ++u) {
+    const int t = wave * kIPW + u;
+    copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
+    c_blk[u] = t * 1024;
+  }
+  auto copy_tiles = [&](char* kdst, char* vdst, int tile_idx) __attribute__((always_inline)) {
+    const int row0 = tile_idx * kTile;
+    const half_t* kp = Kb + (long)row0 * rs;  // wave-uniform
+    const half_t* vp = Vb + (long)row0 * rs;
+    if (row0 + kTile <= N) {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) copy16(kp, c_goff[u], kdst + c_blk[u]);
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) copy16(vp, c_goff[u], vdst + c_blk[u]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) {  // rows past the end re-read row N-1
+        const int back = max(row0 + c_row[u] - (N - 1), 0);
+        copy16(kp, c_goff[u] - back * rs * 2, kdst + c_blk[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) {
+        const int back = max(row0 + c_row[u] - (N - 1), 0);
+        copy16(vp, c_goff[u] - back * rs * 2, vdst + c_blk[u]);
+      }
+    }
+  };
+
+  copy_tiles(k_ring, v_ring, 0);
+  if (nt > 1) copy_tiles(k_ring + T::kBytes, v_ring + T::kBytes, 1);
 
   h8 qf[G::kKSteps], dof[G::kKSteps];
   {
@@ -646,11 +700,9 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   const float l2 = LSE[((long)b * H + h) * N + qrow] * kLog2e;
   const float dl = delta[((long)b * H + h) * N + qrow];
 
-  int nt = (N + kTile - 1) / kTile;
-  if (CAUSAL) nt = min(nt, (min(m0 + kBlockRes, N) - 1) / kTile + 1);
-
-  const int lane_row_off = i * G::kRowBytes + hh * 16;
-  const int lane_tr_off = (4 * hh + ((lane & 15) >> 2)) * G::kRowBytes + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  int r_off[2], c_off[2];
+  swz_rows_off<D>(lane, r_off);
+  swz_cols_off<D>(lane, c_off);
 
   f16v dq[G::kDBlocks];
 #pragma unroll
@@ -658,60 +710,52 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
-  h8 kreg[G::kChunksPerThread], vreg[G::kChunksPerThread];
-  tile_load<D>(Kb, rs, 0, N, kreg);
-  tile_load<D>(Vb, rs, 0, N, vreg);
-  tile_store<D>(smem, kreg);
-  tile_store<D>(smem + G::kTileBytes, vreg);
-  __syncthreads();
+  auto tile = [&](const char* Kl, const char* Vl, int key0, auto masked_tag) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value != 0;
+    h8 dsf[4];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+      f16v s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+      for (int kk = 0; kk < G::kKSteps; ++kk) {
+        s = mfma(swz_rows<D>(Kl, rb, kk, r_off), qf[kk], s);
+        dp = mfma(swz_rows<D>(Vl, rb, kk, r_off), dof[kk], dp);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float p = fast_exp2(fmaf(s[r], c, -l2));
+        if (MASKED) {
+          const int key = key0 + acc_row(rb, r, hh);
+          if ((CAUSAL && key > qi) || key >= N) p = 0.f;
+        }
+        dsf[rb * 2 + (r >> 3)][r & 7] = (half_t)(p * (dp[r] - dl));
+      }
+    }
+#pragma unroll
+    for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db) dq[db] = mfma(swz_cols<D>(Kl, c16, db, c_off), dsf[c16], dq[db]);
+    }
+  };
 
-  for (int kt = 0; kt < nt; ++kt) {
-    const char* Kl = smem + (kt & 1) * 2 * G::kTileBytes;
-    const char* Vl = Kl + G::kTileBytes;
-    const bool more = kt + 1 < nt;
-    if (more) {
-      tile_load<D>(Kb, rs, (kt + 1) * kTile, N, kreg);
-      tile_load<D>(Vb, rs, (kt + 1) * kTile, N, vreg);
+  wait_vm<0>();  // Q, dO rows, lse, delta and the first copies
+  int s0 = 0, s2 = 2;  // j % 3, (j + 2) % 3
+  for (int j = 0; j < nt; ++j) {
+    // tile j was issued two iterations ago; the copies of tile j+1 may still be in flight
+    if (j + 1 < nt) wait_vm<2 * kIPW>();
+    else wait_vm<0>();
+    block_barrier();
+    if (j + 2 < nt) copy_tiles(k_ring + s2 * T::kBytes, v_ring + s2 * T::kBytes, j + 2);
+    if (j < ntw) {
+      const int key0 = j * kTile;
+      const bool masked = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
+      if (masked) tile(k_ring + s0 * T::kBytes, v_ring + s0 * T::kBytes, key0, IntTag<1>{});
+      else tile(k_ring + s0 * T::kBytes, v_ring + s0 * T::kBytes, key0, IntTag<0>{});
     }
-    const int key0 = kt * kTile;
-    const bool active = !CAUSAL || key0 <= q0w + kResident - 1;
-    if (active) {
-      const bool need_mask = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
-      h8 dsf[4];
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-        f16v s, dp;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-        for (int kk = 0; kk < G::kKSteps; ++kk) {
-          s = mfma(read_rows<D>(Kl, rb, kk, lane_row_off), qf[kk], s);
-          dp = mfma(read_rows<D>(Vl, rb, kk, lane_row_off), dof[kk], dp);
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float p = fast_exp2(fmaf(s[r], c, -l2));
-          if (need_mask) {
-            int key = key0 + acc_row(rb, r, hh);
-            if ((CAUSAL && key > qi) || key >= N) p = 0.f;
-          }
-          s[r] = p * (dp[r] - dl);
-        }
-        dsf[rb * 2] = pack8(s, 0);
-        dsf[rb * 2 + 1] = pack8(s, 8);
-      }
-#pragma unroll
-      for (int c16 = 0; c16 < 4; ++c16) {
-#pragma unroll
-        for (int db = 0; db < G::kDBlocks; ++db) dq[db] = mfma(read_cols<D>(Kl, c16, db, lane_tr_off), dsf[c16], dq[db]);
-      }
-    }
-    if (more) {
-      char* Kn = smem + ((kt + 1) & 1) * 2 * G::kTileBytes;
-      tile_store<D>(Kn, kreg);
-      tile_store<D>(Kn + G::kTileBytes, vreg);
-    }
-    __syncthreads();
+    s2 = s0;
+    s0 = s0 == 2 ? 0 : s0 + 1;
   }
   store_resident<D>(dQ + head_off, rs, qi, N, dq, scale, hh);
 }
@@ -1005,9 +1049,10 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
   dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
   const float c = scale * kLog2e;
   if (passes & kPassDq) {
-    fmha_bwd_dq_kernel<D, CAUSAL><<<grid, kThreads, 0, stream>>>(
+    const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;
+    fmha_bwd_dq_kernel<D, CAUSAL><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
         (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
-        (half_t*)dq, head, n, c, scale);
+        (half_t*)dq, head, n, nmb, c, scale);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   if (passes & kPassDkDv) {
