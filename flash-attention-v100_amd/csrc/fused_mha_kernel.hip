@@ -7,7 +7,12 @@
 //   * A wave owns 32 "resident" sequence positions (queries in the forward and
 //     in the dQ pass, keys in the dK/dV pass).  Their rows stay in registers as
 //     MFMA B operands for the whole kernel.  The other sequence dimension is
-//     streamed through LDS in 64-row tiles shared by the 4 waves of a block.
+//     streamed through LDS in 64-row tiles shared by the waves of a block.
+//   * Tiles go global -> LDS with global_load_lds_dwordx4 (no registers in
+//     between) into a 3-slot ring, two tiles ahead of their use; one barrier
+//     per tile.  The LDS layout is XOR-swizzled so that both the row-wise
+//     128-bit reads and the transposing ds_read_b64_tr_b16 reads are free of
+//     bank conflicts without padding.
 //   * The first GEMM is computed transposed, tile^T[streamed][resident], so a
 //     lane holds 16 streamed positions of ONE resident position per 32x32
 //     block.  Row statistics (max, sum, logsumexp, delta) are therefore plain
@@ -15,9 +20,11 @@
 //   * The accumulator registers of the first GEMM, rounded to fp16, are
 //     already laid out as the B operand of the second GEMM, so P and dS never
 //     travel through LDS.  The matching A operand (V^T, K^T, Q^T, dO^T) is read
-//     from the same row-major LDS tile with ds_read_b64_tr_b16.
+//     transposed out of the same row-major tile.
 //   * The backward is split into a dQ pass (query-block parallel) and a dK/dV
 //     pass (key-block parallel): no atomics, no fp32 dQ scratch, deterministic.
+//   * Work-group ids are remapped so that each XCD (private L2) works on whole
+//     (batch, head) slices.
 //
 // Layouts: q/k/v/o/do/dq/dk/dv are (B, N, H, D) fp16, lse/delta are (B, H, N)
 // fp32 (reference: kernel/fused_mha_kernel.cu:57-67).
@@ -37,22 +44,14 @@ typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef short s4 __attribute__((ext_vector_type(4)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef float f4v __attribute__((ext_vector_type(4)));
-typedef float f2v __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 256;      // 4 waves
-constexpr int kWaves = 4;
 constexpr int kResident = 32;      // resident positions per wave
-constexpr int kBlockRes = kWaves * kResident;  // 128 resident positions per block
 constexpr int kTile = 64;          // streamed rows per LDS tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
 template <int D>
 struct TileGeom {
-  static constexpr int kRowBytes = D * 2 + 16;             // padded LDS row
-  static constexpr int kTileBytes = kTile * kRowBytes;
-  static constexpr int kChunksPerRow = D / 8;              // 16-byte chunks
-  static constexpr int kChunksPerThread = kTile * kChunksPerRow / kThreads;
   static constexpr int kKSteps = D / 16;                   // MFMA k-steps over D
   static constexpr int kDBlocks = D / 32;                  // 32-row blocks over D
 };
@@ -70,62 +69,6 @@ __device__ __forceinline__ float other_half(float x) {
   // r[0]: lanes 0-31 keep own, lanes 32-63 get lane-32's; r[1] the converse.
   int mine_or_other = (threadIdx.x & 32) ? r[0] : r[1];
   return __int_as_float(mine_or_other);
-}
-
-// Global -> registers for one 64-row tile (rows clamped to n-1).
-template <int D>
-__device__ __forceinline__ void tile_load(const half_t* __restrict__ base, long row_stride,
-                                          int row0, int n, h8 (&regs)[TileGeom<D>::kChunksPerThread]) {
-  using G = TileGeom<D>;
-#pragma unroll
-  for (int i = 0; i < G::kChunksPerThread; ++i) {
-    int ch = threadIdx.x + kThreads * i;
-    int r = ch / G::kChunksPerRow;
-    int c = ch % G::kChunksPerRow;
-    int row = min(row0 + r, n - 1);
-    regs[i] = *reinterpret_cast<const h8*>(base + (long)row * row_stride + c * 8);
-  }
-}
-
-// Registers -> LDS (row-major, padded rows).
-template <int D>
-__device__ __forceinline__ void tile_store(char* lds, const h8 (&regs)[TileGeom<D>::kChunksPerThread]) {
-  using G = TileGeom<D>;
-#pragma unroll
-  for (int i = 0; i < G::kChunksPerThread; ++i) {
-    int ch = threadIdx.x + kThreads * i;
-    int r = ch / G::kChunksPerRow;
-    int c = ch % G::kChunksPerRow;
-    *reinterpret_cast<h8*>(lds + r * G::kRowBytes + c * 16) = regs[i];
-  }
-}
-
-// A operand of the first GEMM: rows = 32 streamed positions (row-block rb),
-// k = 16 feature columns of k-step kk.  Lane (i, hh) reads 8 contiguous halves.
-template <int D>
-__device__ __forceinline__ h8 read_rows(const char* lds, int rb, int kk, int lane_row_off) {
-  return *reinterpret_cast<const h8*>(lds + lane_row_off + rb * 32 * TileGeom<D>::kRowBytes + kk * 32);
-}
-
-// A operand of the second GEMM: rows = 32 feature columns (block db), k = 16
-// streamed positions of chunk c16, read transposed out of the row-major tile.
-// The k order matches the accumulator layout of the first GEMM:
-// k index 8*hh + j  <->  streamed row 16*c16 + 8*(j/4) + 4*hh + j%4.
-template <int D>
-__device__ __forceinline__ h8 read_cols(const char* lds, int c16, int db, int lane_tr_off) {
-  using G = TileGeom<D>;
-  typedef __attribute__((address_space(3))) s4 lds_s4;
-  const char* p = lds + lane_tr_off + c16 * 16 * G::kRowBytes + db * 64;
-  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p));
-  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + 8 * G::kRowBytes));
-  return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-}
-
-__device__ __forceinline__ h8 pack8(const f16v& x, int base) {
-  h8 r;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) r[j] = (half_t)x[base + j];
-  return r;
 }
 
 // Streamed-row index of accumulator register r in row-block rb for half hh.
@@ -151,75 +94,6 @@ __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long r
       *reinterpret_cast<h4*>(p + db * 32 + 8 * g + 4 * hh) = v;
     }
   }
-}
-
-// ---------------------------------------------------------------------------
-// Streaming of 64-row tiles, global -> registers -> LDS, with per-thread
-// offsets computed once.  PAD is the padding of an LDS row in bytes: 16 makes
-// the 128-bit row reads conflict-free, 32 the transposed 64-bit reads.
-// ---------------------------------------------------------------------------
-template <int D, int PAD>
-struct TileStream {
-  static constexpr int kRowBytes = D * 2 + PAD;
-  static constexpr int kTileBytes = kTile * kRowBytes;
-  static constexpr int kCPT = TileGeom<D>::kChunksPerThread;
-  int goff[kCPT];  // element offset of this thread's chunks inside a full tile
-  int loff[kCPT];  // byte offset inside the LDS tile
-  int row[kCPT];
-  int col[kCPT];
-
-  __device__ __forceinline__ void init(int row_stride) {
-#pragma unroll
-    for (int i = 0; i < kCPT; ++i) {
-      int ch = threadIdx.x + kThreads * i;
-      row[i] = ch / TileGeom<D>::kChunksPerRow;
-      col[i] = (ch % TileGeom<D>::kChunksPerRow) * 8;
-      goff[i] = row[i] * row_stride + col[i];
-      loff[i] = row[i] * kRowBytes + col[i] * 2;
-    }
-  }
-  // `base` points at row 0 of the (batch, head) slice; rows past n-1 are clamped.
-  __device__ __forceinline__ void load(const half_t* __restrict__ base, int row_stride, int row0, int n,
-                                       h8 (&regs)[kCPT]) const {
-    const half_t* tile = base + (long)row0 * row_stride;  // wave-uniform
-    if (row0 + kTile <= n) {
-#pragma unroll
-      for (int i = 0; i < kCPT; ++i) regs[i] = *reinterpret_cast<const h8*>(tile + goff[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < kCPT; ++i) {
-        int r = min(row0 + row[i], n - 1);
-        regs[i] = *reinterpret_cast<const h8*>(base + (long)r * row_stride + col[i]);
-      }
-    }
-  }
-  __device__ __forceinline__ void store(char* lds, const h8 (&regs)[kCPT]) const {
-#pragma unroll
-    for (int i = 0; i < kCPT; ++i) *reinterpret_cast<h8*>(lds + loff[i]) = regs[i];
-  }
-};
-
-// Lane-constant byte offsets of the two LDS read patterns.
-template <int ROWB>
-__device__ __forceinline__ int lane_rows_off(int lane) { return (lane & 31) * ROWB + (lane >> 5) * 16; }
-template <int ROWB>
-__device__ __forceinline__ int lane_cols_off(int lane) {
-  return (4 * (lane >> 5) + ((lane & 15) >> 2)) * ROWB + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-}
-// A operand, rows = 32 streamed positions of row-block rb, k = features of k-step kk.
-template <int ROWB>
-__device__ __forceinline__ h8 lds_rows(const char* lds, int rb, int kk, int lane_off) {
-  return *reinterpret_cast<const h8*>(lds + lane_off + rb * 32 * ROWB + kk * 32);
-}
-// A operand, rows = 32 features of block db, k = streamed positions of chunk c16
-// in accumulator order (k index 8*hh + j <-> row 16*c16 + 8*(j/4) + 4*hh + j%4).
-template <int ROWB>
-__device__ __forceinline__ h8 lds_cols(const char* lds, int c16, int db, int lane_off) {
-  typedef __attribute__((address_space(3))) s4 lds_s4;
-  const char* p = lds + lane_off + c16 * 16 * ROWB + db * 64;
-  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p));
-  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + 8 * ROWB));
-  return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
 // Sum of the 8 halves of x added to acc, two at a time (v_dot2_f32_f16).
@@ -1046,7 +920,6 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
         (const half_t*)o, (const half_t*)d_o, (const float*)lse, delta, delta + (long)batch * head * n, head, n, rows);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
-  dim3 grid((n + kBlockRes - 1) / kBlockRes, batch * head);
   const float c = scale * kLog2e;
   if (passes & kPassDq) {
     const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;

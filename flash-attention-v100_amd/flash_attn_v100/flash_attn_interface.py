@@ -55,7 +55,8 @@ class FlashAttnFunc(torch.autograd.Function):
         q, k, v, out, softmax_lse = ctx.saved_tensors
         # every element of dq, dk, dv is written by the kernels: no zero fill
         # (the reference needs zeros for its atomics, :84)
-        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        # dense (B, N, H, D) whatever the strides of the saved inputs are
+        dq, dk, dv = (torch.empty_like(x, memory_format=torch.contiguous_format) for x in (q, k, v))
         _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, ctx.softmax_scale, ctx.causal)
         return dq, dk, dv, None, None
 
