@@ -147,6 +147,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy three times (reference point for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus)
@@ -158,6 +160,14 @@ def main():
     props = torch.cuda.get_device_properties(0)
     clock_ghz = props.clock_rate / 1e6 if hasattr(props, "clock_rate") else 2.4
     peak_check = props.multi_processor_count * 4 * 1024 * clock_ghz / 1e3  # CUs x SIMDs x flop/clk x GHz
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     name, B, H, N, D, causal = CONFIGS[HEADLINE]
     q, k, v, do = make_device_inputs(B, H, N, D)
