@@ -635,21 +635,23 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 }
 
 // ---------------------------------------------------------------------------
-// Backward, dK/dV pass.  Block = 4 waves = 128 keys, wave = 32 keys, one wave
-// per SIMD (the wave keeps K, V rows and the dK, dV accumulators of its keys in
-// registers); Q/dO tiles of 64 queries stream through a 3-slot LDS ring, copied
-// asynchronously two tiles ahead, together with the tile's lse and delta rows.
-//   S = Q K^T, dP = dO V^T, P = exp(S - lse), dS = P o (dP - delta),
-//   dV^T += dO^T P, dK^T += Q^T dS
+// Backward, dK/dV pass.  Block = 128 keys = 4 pairs of waves; a pair owns 32
+// keys and splits the work so that each wave keeps only one accumulator and one
+// of K / V in registers (two waves per SIMD fit):
+//   wave A (waves 0-3): S = Q K^T, P = exp(S - lse)   -> P to LDS,  dV^T += dO^T P
+//   wave B (waves 4-7): dP = dO V^T, T = dP - delta   <- P from LDS, dS = P o T,
+//                                                      dK^T += Q^T dS
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 618-629, 653-656,
-// 697-712; key-block-parallel launch as at :908-915).
+// 697-712; key-block-parallel launch as at :908-915).  P travels in the
+// accumulator layout, lane for lane, so no transposition is involved.  Q/dO
+// tiles of 64 queries stream through a 3-slot LDS ring, copied two tiles
+// ahead, with the tile's lse2 and delta rows.  Two barriers per tile: one for
+// the tile, one for P.
 // ---------------------------------------------------------------------------
-#ifndef KV_HINTS
-#define KV_HINTS 1
-#endif
-constexpr int kKvWaves = 4;
+constexpr int kKvPairs = 4;
+constexpr int kKvWaves = 2 * kKvPairs;
 constexpr int kKvThreads = kKvWaves * 64;
-constexpr int kKvBlockKeys = kKvWaves * kResident;
+constexpr int kKvBlockKeys = kKvPairs * kResident;
 
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(kKvThreads, 1)
@@ -659,19 +661,20 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kKvWaves;  // copies per wave per tile, per tensor
-  constexpr int kPerIter = 2 * kIPW + 1;       // Q, dO and one lse/delta copy
-  static_assert(kPerIter < 16, "vmcnt immediate");
-  // Q ring, dO ring, then per slot and wave 64 lse2 values followed by 64 delta
-  // values (and 512 bytes unused).  Slots are addressed at run time; the copies
-  // into them are inline asm (see copy16).
-  __shared__ __attribute__((aligned(1024))) char smem[3 * (2 * T::kBytes + kKvWaves * 1024)];
+  // Q ring, dO ring, per slot 64 lse2 then 64 delta values (1 KiB, half unused),
+  // and the P exchange: per pair two 32x32 fp16 blocks, 32 bytes per lane each.
+  constexpr int kStBytes = 1024;
+  constexpr int kPBytes = kKvPairs * 2 * 2048;
+  __shared__ __attribute__((aligned(1024))) char smem[3 * (2 * T::kBytes + kStBytes) + kPBytes];
   char* const q_ring = smem;
   char* const g_ring = smem + 3 * T::kBytes;
   char* const st_ring = smem + 6 * T::kBytes;
-  constexpr int kStBytes = kKvWaves * 1024;
+  char* const p_xchg = st_ring + 3 * kStBytes;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pair = wave & (kKvPairs - 1);
+  const bool role_b = wave >= kKvPairs;
   const int i = lane & 31, hh = lane >> 5;
   int bh, nblk;
   slice_and_block(nnb, bh, nblk);  // causal: low key blocks are the heavy ones and come first
@@ -684,7 +687,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   const int lse2_off = (int)(lse2 - delta) * 4;  // bytes from the delta row to the lse2 row; lse2 lies behind delta
 
   const int n0 = nblk * kKvBlockKeys;
-  const int k0w = n0 + wave * kResident;
+  const int k0w = n0 + pair * kResident;
   const int ki = k0w + i;
   const int krow = min(ki, N - 1);
 
@@ -700,14 +703,16 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
     c_blk[u] = t * 1024;
   }
-  // lse/delta copy: lanes 0-15 fetch the tile's 64 lse values, lanes 16-31 its
-  // 64 delta values, 4 floats each; lanes 32-63 repeat them into unused space.
+  // lse2/delta copy (wave 0 only): lanes 0-15 fetch the tile's 64 lse2 values, lanes
+  // 16-31 its 64 delta values, 4 floats each; lanes 32-63 repeat them into unused space.
   const int st_quad = (lane & 15) * 4;
   const bool st_is_delta = (lane >> 4) & 1;
-  auto copy_tiles = [&](char* qdst, char* gdst, char* sdst, int tile_idx) __attribute__((always_inline)) {
+  auto copy_tiles = [&](int slot, int tile_idx) __attribute__((always_inline)) {
     const int row0 = tile_idx * kTile;
     const half_t* qp = Qb + (long)row0 * rs;   // wave-uniform
     const half_t* gp = dOb + (long)row0 * rs;
+    char* qdst = q_ring + slot * T::kBytes;
+    char* gdst = g_ring + slot * T::kBytes;
     if (row0 + kTile <= N) {
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) copy16(qp, c_goff[u], qdst + c_blk[u]);
@@ -725,161 +730,153 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
         copy16(gp, c_goff[u] - back * rs * 2, gdst + c_blk[u]);
       }
     }
-    // N is a multiple of 32, so a quad of rows is either inside or outside [0, N)
-    const int quad = min(row0 + st_quad, N - 4);
-    copy16(reinterpret_cast<const half_t*>(delta_b), quad * 4 + (st_is_delta ? 0 : lse2_off), sdst + wave * 1024);
+    if (wave == 0) {
+      // N is a multiple of 32, so a quad of rows is either inside or outside [0, N)
+      const int quad = min(row0 + st_quad, N - 4);
+      copy16(reinterpret_cast<const half_t*>(delta_b), quad * 4 + (st_is_delta ? 0 : lse2_off),
+             st_ring + slot * kStBytes);
+    }
   };
 
-  copy_tiles(q_ring, g_ring, st_ring, t_begin);
-  if (n_it > 1) copy_tiles(q_ring + T::kBytes, g_ring + T::kBytes, st_ring + kStBytes, t_begin + 1);
+  copy_tiles(0, t_begin);
+  if (n_it > 1) copy_tiles(1, t_begin + 1);
 
-  h8 kf[G::kKSteps], vf[G::kKSteps];
+  // resident rows of this wave: K for role A, V for role B
+  h8 rf[G::kKSteps];
   {
-    const half_t* kp = K + head_off + (long)krow * rs + hh * 8;
-    const half_t* vp = V + head_off + (long)krow * rs + hh * 8;
+    const half_t* rp = (role_b ? V : K) + head_off + (long)krow * rs + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) {
-      kf[kk] = *reinterpret_cast<const h8*>(kp + kk * 16);
-      vf[kk] = *reinterpret_cast<const h8*>(vp + kk * 16);
-    }
+    for (int kk = 0; kk < G::kKSteps; ++kk) rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
   }
 
   int r_off[2], c_off[2];
   swz_rows_off<D>(lane, r_off);
   swz_cols_off<D>(lane, c_off);
-  const int st_off = wave * 1024 + hh * 16;  // + (rb * 32 + 8 * g) * 4: lse quad; + 256: delta quad
+  const int st_off = hh * 16 + (role_b ? 256 : 0);   // + (rb * 32 + 8 * g) * 4: this role's quad
+  char* const p_mine = p_xchg + pair * 4096 + lane * 32;  // + rb * 2048
 
-  f16v dk[G::kDBlocks], dv[G::kDBlocks];
+  f16v acc[G::kDBlocks];  // dV^T (role A) or dK^T (role B)
 #pragma unroll
   for (int db = 0; db < G::kDBlocks; ++db)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { dk[db][r] = 0.f; dv[db][r] = 0.f; }
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
 
-  // One 64-query tile.  MASKED tiles straddle the diagonal or the end of the sequence.
-  // Written as four MFMA stretches (scores of both 32-query halves, then the two
-  // gradient updates) with the element-wise work of a half placed next to an MFMA
-  // stretch that does not depend on it, all in one basic block, so the scheduler
-  // can run VALU work in the shadow of MFMAs.
-  auto tile = [&](const char* Ql, const char* Gl, const char* Sl, int q0, auto masked_tag) __attribute__((always_inline)) {
-    constexpr bool MASKED = decltype(masked_tag)::value != 0;
-    f16v s[2], dp[2];
-    h8 pf[2][2], dsf[2][2];
-    auto gemm1 = [&](int rb) __attribute__((always_inline)) {
+  // first GEMM of a tile: rows of Q (role A) or dO (role B) against the resident rows
+  auto gemm1 = [&](const char* tile_lds, f16v (&x)[2]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[rb][r] = 0.f; dp[rb][r] = 0.f; }
+    for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-      for (int kk = 0; kk < G::kKSteps; ++kk) {
-        s[rb] = mfma(swz_rows<D>(Ql, rb, kk, r_off), kf[kk], s[rb]);
-        dp[rb] = mfma(swz_rows<D>(Gl, rb, kk, r_off), vf[kk], dp[rb]);
-      }
-    };
-    auto pointwise = [&](int rb) __attribute__((always_inline)) {
+      for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f4v l4 = *reinterpret_cast<const f4v*>(Sl + st_off + (rb * 32 + 8 * g) * 4);
-        const f4v d4 = *reinterpret_cast<const f4v*>(Sl + st_off + 256 + (rb * 32 + 8 * g) * 4);
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * g + e;
-          float p = fast_exp2(fmaf(s[rb][r], c, -l4[e]));
-          if (MASKED) {
-            const int q = q0 + rb * 32 + 8 * g + 4 * hh + e;
-            if ((CAUSAL && ki > q) || q >= N) p = 0.f;
-          }
-          const float ds = p * (dp[rb][r] - d4[e]);
-          pf[rb][g >> 1][(g & 1) * 4 + e] = (half_t)p;
-          dsf[rb][g >> 1][(g & 1) * 4 + e] = (half_t)ds;
-        }
-      }
-    };
-    auto gemm2 = [&](int rb) __attribute__((always_inline)) {
-#pragma unroll
-      for (int cc = 0; cc < 2; ++cc) {
-        const int c16 = rb * 2 + cc;
-#pragma unroll
-        for (int db = 0; db < G::kDBlocks; ++db) {
-          dv[db] = mfma(swz_cols<D>(Gl, c16, db, c_off), pf[rb][cc], dv[db]);
-          dk[db] = mfma(swz_cols<D>(Ql, c16, db, c_off), dsf[rb][cc], dk[db]);
-        }
-      }
-    };
-    gemm1(0);
-    gemm1(1);
-    pointwise(0);
-    gemm2(0);
-    pointwise(1);
-    gemm2(1);
-#if KV_HINTS == 2
-    // Order for the scheduler (masks: 0x008 MFMA, 0x100 LDS read, 0x002 VALU):
-    // LDS reads run ahead of the MFMAs that use them, and the element-wise work of
-    // half 0 / half 1 is spread over the MFMAs of gemm1(1) / gemm2(0).
-    constexpr int kM = 2 * G::kKSteps;  // MFMAs per gemm1 half == per gemm2 half
-    constexpr int kLead = 4;
-    constexpr int kValuPerMfma = 7;
+      for (int rb = 0; rb < 2; ++rb) x[rb] = mfma(swz_rows<D>(tile_lds, rb, kk, r_off), rf[kk], x[rb]);
+    }
+    constexpr int kN = 2 * G::kKSteps, kLead = 4;
     __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
 #pragma unroll
-    for (int n = 0; n < kM; ++n) {  // gemm1(0); its reads continue into gemm1(1)
+    for (int n = 0; n < kN - kLead; ++n) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // lse / delta of half 0
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
+  };
+  // second GEMM: columns of dO (role A) or Q (role B) against the fp16 operand y
+  auto gemm2 = [&](const char* tile_lds, const h8 (&y)[4]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int n = 0; n < kM; ++n) {  // gemm1(1) with pointwise(0)
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (n < kM - kLead) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
+    for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db) acc[db] = mfma(swz_cols<D>(tile_lds, c16, db, c_off), y[c16], acc[db]);
     }
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead + 8, 0);  // first gemm2 operands, lse / delta of half 1
+    constexpr int kN = 4 * G::kDBlocks, kLead = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead, 0);
 #pragma unroll
-    for (int n = 0; n < kM; ++n) {  // gemm2(0) with pointwise(1)
+    for (int n = 0; n < kN - kLead; ++n) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
     }
-#pragma unroll
-    for (int n = 0; n < kM; ++n) {  // gemm2(1)
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (n < kM - kLead) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-#elif KV_HINTS == 1
-    // LDS reads run kLead MFMAs ahead of their use inside each MFMA stretch.
-    constexpr int kM1 = 4 * G::kKSteps, kM2 = 4 * G::kKSteps, kLead1 = 4;
-    __builtin_amdgcn_sched_group_barrier(0x100, kLead1, 0);
-#pragma unroll
-    for (int n = 0; n < kM1 - kLead1; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kLead1, 0);
-    (void)kM2;
-#endif
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
 
-  wait_vm<0>();  // K/V rows and the first copies: nothing is left for the compiler to wait on in the loop
+  wait_vm<0>();  // resident rows and the first copies: nothing is left for the compiler to wait on in the loop
   int s0 = 0, s2 = 2;  // it % 3, (it + 2) % 3
   for (int it = 0; it < n_it; ++it) {
     // tile `it` was issued two iterations ago; the copies of tile it+1 may still be in flight
-    if (it + 1 < n_it) wait_vm<kPerIter>();
-    else wait_vm<0>();
+    if (it + 1 < n_it) {
+      if (wave == 0) wait_vm<2 * kIPW + 1>();
+      else wait_vm<2 * kIPW>();
+    } else {
+      wait_vm<0>();
+    }
     block_barrier();
-    if (it + 2 < n_it)
-      copy_tiles(q_ring + s2 * T::kBytes, g_ring + s2 * T::kBytes, st_ring + s2 * kStBytes, t_begin + it + 2);
+    if (it + 2 < n_it) copy_tiles(s2, t_begin + it + 2);
     const char* Ql = q_ring + s0 * T::kBytes;
     const char* Gl = g_ring + s0 * T::kBytes;
-    const char* Sl = st_ring + s0 * kStBytes;
+    const char* Sl = st_ring + s0 * kStBytes + st_off;
     const int q0 = (t_begin + it) * kTile;
     const bool active = !CAUSAL || q0 + kTile - 1 >= k0w;
+    const bool masked = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
+    h8 y[4];      // role A: P, role B: dS, fp16 in B-operand order
+    f16v x[2];    // role A: S, role B: dP - delta
     if (active) {
-      const bool masked = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
-      if (masked) tile(Ql, Gl, Sl, q0, IntTag<1>{});
-      else tile(Ql, Gl, Sl, q0, IntTag<0>{});
+      if (!role_b) {
+        gemm1(Ql, x);
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f4v l4 = *reinterpret_cast<const f4v*>(Sl + (rb * 32 + 8 * g) * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              float p = fast_exp2(fmaf(x[rb][4 * g + e], c, -l4[e]));
+              if (masked) {
+                const int q = q0 + rb * 32 + 8 * g + 4 * hh + e;
+                if ((CAUSAL && ki > q) || q >= N) p = 0.f;
+              }
+              y[rb * 2 + (g >> 1)][(g & 1) * 4 + e] = (half_t)p;
+            }
+          }
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+          *reinterpret_cast<h8*>(p_mine + rb * 2048) = y[rb * 2];
+          *reinterpret_cast<h8*>(p_mine + rb * 2048 + 16) = y[rb * 2 + 1];
+        }
+      } else {
+        gemm1(Gl, x);
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f4v d4 = *reinterpret_cast<const f4v*>(Sl + (rb * 32 + 8 * g) * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[rb][4 * g + e] -= d4[e];
+          }
+      }
+    }
+    block_barrier();  // P of this tile is in LDS
+    if (active) {
+      if (!role_b) {
+        gemm2(Gl, y);
+      } else {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+          const h8 p0 = *reinterpret_cast<const h8*>(p_mine + rb * 2048);
+          const h8 p1 = *reinterpret_cast<const h8*>(p_mine + rb * 2048 + 16);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
+            y[rb * 2 + 1][e] = (half_t)((float)p1[e] * x[rb][8 + e]);
+          }
+        }
+        gemm2(Ql, y);
+      }
     }
     s2 = s0;
     s0 = s0 == 2 ? 0 : s0 + 1;
   }
 
-  store_resident<D>(dK + head_off, rs, ki, N, dk, scale, hh);
-  store_resident<D>(dV + head_off, rs, ki, N, dv, 1.f, hh);
+  if (!role_b) store_resident<D>(dV + head_off, rs, ki, N, acc, 1.f, hh);
+  else store_resident<D>(dK + head_off, rs, ki, N, acc, scale, hh);
 }
 
 // ---------------------------------------------------------------------------
