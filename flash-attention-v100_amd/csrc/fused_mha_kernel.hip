@@ -481,15 +481,22 @@ fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ d
 }
 
 // ---------------------------------------------------------------------------
-// Backward, dQ pass.  Block = 8 waves = 256 queries, wave = 32 queries; K/V
-// tiles of 64 keys stream through a 3-slot LDS ring, copied two tiles ahead.
-//   S^T = K Q^T, dP^T = V dO^T, dS^T = P^T o (dP^T - delta), dQ^T += K^T dS^T
+// Backward, dQ pass.  Block = 128 queries = 4 pairs of waves; a pair owns 32
+// queries and splits the work (two waves per SIMD fit):
+//   wave A (waves 0-3): S^T = K Q^T, P^T = exp(S^T - lse)   -> P^T to LDS
+//   wave B (waves 4-7): dP^T = V dO^T, T = dP^T - delta      <- P^T from LDS,
+//                       dS^T = P^T o T                       -> dS^T to LDS
+//   both:               dQ^T += K^T dS^T, each for half of the head dimension
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 653-656, 680-683).
 // lse and delta belong to the resident query, so they are per-lane scalars.
+// P^T and dS^T travel in the accumulator layout, lane for lane.  K/V tiles of 64
+// keys stream through a 3-slot LDS ring, copied two tiles ahead.  Three barriers
+// per tile: the tile, P^T, dS^T.
 // ---------------------------------------------------------------------------
-constexpr int kDqWaves = 4;
+constexpr int kDqPairs = 4;
+constexpr int kDqWaves = 2 * kDqPairs;
 constexpr int kDqThreads = kDqWaves * 64;
-constexpr int kDqBlockQ = kDqWaves * kResident;
+constexpr int kDqBlockQ = kDqPairs * kResident;
 
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(kDqThreads, 1)
@@ -499,12 +506,19 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kDqWaves;  // copies per wave per tile, per tensor
-  __shared__ __attribute__((aligned(1024))) char smem[2 * 3 * T::kBytes];  // K ring, V ring
+  constexpr int kHalfDB = G::kDBlocks / 2;     // 32-feature blocks of dQ per wave
+  // K ring, V ring, then per pair a 64x32 fp16 block (32 x 2 x 32 bytes per lane ... 4 KiB) for P^T and one for dS^T
+  constexpr int kXBytes = kDqPairs * 4096;
+  __shared__ __attribute__((aligned(1024))) char smem[2 * 3 * T::kBytes + 2 * kXBytes];
   char* const k_ring = smem;
   char* const v_ring = smem + 3 * T::kBytes;
+  char* const p_xchg = smem + 6 * T::kBytes;
+  char* const ds_xchg = p_xchg + kXBytes;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int pair = wave & (kDqPairs - 1);
+  const bool role_b = wave >= kDqPairs;
   const int i = lane & 31, hh = lane >> 5;
   int bh, mb;
   slice_and_block(nmb, bh, mb);
@@ -516,7 +530,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   const half_t* Vb = V + head_off;
 
   const int m0 = mblk * kDqBlockQ;
-  const int q0w = m0 + wave * kResident;
+  const int q0w = m0 + pair * kResident;
   const int qi = q0w + i;
   const int qrow = min(qi, N - 1);
 
@@ -535,10 +549,12 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
     copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
     c_blk[u] = t * 1024;
   }
-  auto copy_tiles = [&](char* kdst, char* vdst, int tile_idx) __attribute__((always_inline)) {
+  auto copy_tiles = [&](int slot, int tile_idx) __attribute__((always_inline)) {
     const int row0 = tile_idx * kTile;
     const half_t* kp = Kb + (long)row0 * rs;  // wave-uniform
     const half_t* vp = Vb + (long)row0 * rs;
+    char* kdst = k_ring + slot * T::kBytes;
+    char* vdst = v_ring + slot * T::kBytes;
     if (row0 + kTile <= N) {
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) copy16(kp, c_goff[u], kdst + c_blk[u]);
@@ -558,80 +574,138 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
     }
   };
 
-  copy_tiles(k_ring, v_ring, 0);
-  if (nt > 1) copy_tiles(k_ring + T::kBytes, v_ring + T::kBytes, 1);
+  copy_tiles(0, 0);
+  if (nt > 1) copy_tiles(1, 1);
 
-  h8 qf[G::kKSteps], dof[G::kKSteps];
+  // resident rows of this wave: Q for role A, dO for role B; and the row statistic it needs
+  h8 rf[G::kKSteps];
   {
-    const half_t* qp = Q + head_off + (long)qrow * rs + hh * 8;
-    const half_t* gp = dO + head_off + (long)qrow * rs + hh * 8;
+    const half_t* rp = (role_b ? dO : Q) + head_off + (long)qrow * rs + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) {
-      qf[kk] = *reinterpret_cast<const h8*>(qp + kk * 16);
-      dof[kk] = *reinterpret_cast<const h8*>(gp + kk * 16);
-    }
+    for (int kk = 0; kk < G::kKSteps; ++kk) rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
   }
-  const float l2 = LSE[((long)b * H + h) * N + qrow] * kLog2e;
-  const float dl = delta[((long)b * H + h) * N + qrow];
+  const long stat_at = ((long)b * H + h) * N + qrow;
+  const float stat = role_b ? delta[stat_at] : LSE[stat_at] * kLog2e;
 
   int r_off[2], c_off[2];
   swz_rows_off<D>(lane, r_off);
   swz_cols_off<D>(lane, c_off);
+  char* const p_mine = p_xchg + pair * 4096 + lane * 32;    // + rb * 2048
+  char* const ds_mine = ds_xchg + pair * 4096 + lane * 32;  // + rb * 2048
+  const int db0 = role_b ? kHalfDB : 0;  // first 32-feature block of dQ this wave accumulates
 
-  f16v dq[G::kDBlocks];
+  f16v dq[kHalfDB];
 #pragma unroll
-  for (int db = 0; db < G::kDBlocks; ++db)
+  for (int db = 0; db < kHalfDB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
-  auto tile = [&](const char* Kl, const char* Vl, int key0, auto masked_tag) __attribute__((always_inline)) {
-    constexpr bool MASKED = decltype(masked_tag)::value != 0;
-    h8 dsf[4];
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb) {
-      f16v s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
-#pragma unroll
-      for (int kk = 0; kk < G::kKSteps; ++kk) {
-        s = mfma(swz_rows<D>(Kl, rb, kk, r_off), qf[kk], s);
-        dp = mfma(swz_rows<D>(Vl, rb, kk, r_off), dof[kk], dp);
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float p = fast_exp2(fmaf(s[r], c, -l2));
-        if (MASKED) {
-          const int key = key0 + acc_row(rb, r, hh);
-          if ((CAUSAL && key > qi) || key >= N) p = 0.f;
-        }
-        dsf[rb * 2 + (r >> 3)][r & 7] = (half_t)(p * (dp[r] - dl));
-      }
-    }
-#pragma unroll
-    for (int c16 = 0; c16 < 4; ++c16) {
-#pragma unroll
-      for (int db = 0; db < G::kDBlocks; ++db) dq[db] = mfma(swz_cols<D>(Kl, c16, db, c_off), dsf[c16], dq[db]);
-    }
-  };
-
-  wait_vm<0>();  // Q, dO rows, lse, delta and the first copies
+  wait_vm<0>();  // resident rows, statistics and the first copies
   int s0 = 0, s2 = 2;  // j % 3, (j + 2) % 3
   for (int j = 0; j < nt; ++j) {
     // tile j was issued two iterations ago; the copies of tile j+1 may still be in flight
     if (j + 1 < nt) wait_vm<2 * kIPW>();
     else wait_vm<0>();
     block_barrier();
-    if (j + 2 < nt) copy_tiles(k_ring + s2 * T::kBytes, v_ring + s2 * T::kBytes, j + 2);
-    if (j < ntw) {
-      const int key0 = j * kTile;
-      const bool masked = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
-      if (masked) tile(k_ring + s0 * T::kBytes, v_ring + s0 * T::kBytes, key0, IntTag<1>{});
-      else tile(k_ring + s0 * T::kBytes, v_ring + s0 * T::kBytes, key0, IntTag<0>{});
+    if (j + 2 < nt) copy_tiles(s2, j + 2);
+    const char* Kl = k_ring + s0 * T::kBytes;
+    const char* Vl = v_ring + s0 * T::kBytes;
+    const bool active = j < ntw;
+    const int key0 = j * kTile;
+    const bool masked = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
+    f16v x[2];  // role A: S^T, role B: dP^T - delta
+    if (active) {
+      const char* tl = role_b ? Vl : Kl;
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < G::kKSteps; ++kk) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) x[rb] = mfma(swz_rows<D>(tl, rb, kk, r_off), rf[kk], x[rb]);
+      }
+      {
+        constexpr int kN = 2 * G::kKSteps, kLead = 4;
+        __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
+#pragma unroll
+        for (int n = 0; n < kN - kLead; ++n) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
+      }
+      if (!role_b) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+          h8 y0, y1;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float p = fast_exp2(fmaf(x[rb][r], c, -stat));
+            if (masked) {
+              const int key = key0 + acc_row(rb, r, hh);
+              if ((CAUSAL && key > qi) || key >= N) p = 0.f;
+            }
+            if (r < 8) y0[r] = (half_t)p; else y1[r - 8] = (half_t)p;
+          }
+          *reinterpret_cast<h8*>(p_mine + rb * 2048) = y0;
+          *reinterpret_cast<h8*>(p_mine + rb * 2048 + 16) = y1;
+        }
+      } else {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) x[rb][r] -= stat;
+      }
+    }
+    block_barrier();  // P^T of this tile is in LDS
+    if (active && role_b) {
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        const h8 p0 = *reinterpret_cast<const h8*>(p_mine + rb * 2048);
+        const h8 p1 = *reinterpret_cast<const h8*>(p_mine + rb * 2048 + 16);
+        h8 y0, y1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          y0[e] = (half_t)((float)p0[e] * x[rb][e]);
+          y1[e] = (half_t)((float)p1[e] * x[rb][8 + e]);
+        }
+        *reinterpret_cast<h8*>(ds_mine + rb * 2048) = y0;
+        *reinterpret_cast<h8*>(ds_mine + rb * 2048 + 16) = y1;
+      }
+    }
+    block_barrier();  // dS^T of this tile is in LDS
+    if (active) {
+      h8 y[4];
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        y[rb * 2] = *reinterpret_cast<const h8*>(ds_mine + rb * 2048);
+        y[rb * 2 + 1] = *reinterpret_cast<const h8*>(ds_mine + rb * 2048 + 16);
+      }
+#pragma unroll
+      for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+        for (int db = 0; db < kHalfDB; ++db) dq[db] = mfma(swz_cols<D>(Kl, c16, db0 + db, c_off), y[c16], dq[db]);
+      }
     }
     s2 = s0;
     s0 = s0 == 2 ? 0 : s0 + 1;
   }
-  store_resident<D>(dQ + head_off, rs, qi, N, dq, scale, hh);
+
+  // each wave of the pair stores its half of the head dimension
+  if (qi < N) {
+    half_t* op = dQ + head_off + (long)qi * rs + db0 * 32;
+#pragma unroll
+    for (int db = 0; db < kHalfDB; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        h4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (half_t)(dq[db][4 * g + e] * scale);
+        *reinterpret_cast<h4*>(op + db * 32 + 8 * g + 4 * hh) = v;
+      }
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
