@@ -507,13 +507,13 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kDqWaves;  // copies per wave per tile, per tensor
   constexpr int kHalfDB = G::kDBlocks / 2;     // 32-feature blocks of dQ per wave
-  // K ring, V ring, then per pair a 64x32 fp16 block (32 x 2 x 32 bytes per lane ... 4 KiB) for P^T and one for dS^T
+  // K ring, V ring, then per pair a 64x32 fp16 block (4 KiB) holding P^T and later dS^T
   constexpr int kXBytes = kDqPairs * 4096;
-  __shared__ __attribute__((aligned(1024))) char smem[2 * 3 * T::kBytes + 2 * kXBytes];
+  __shared__ __attribute__((aligned(1024))) char smem[2 * 3 * T::kBytes + kXBytes];
   char* const k_ring = smem;
   char* const v_ring = smem + 3 * T::kBytes;
   char* const p_xchg = smem + 6 * T::kBytes;
-  char* const ds_xchg = p_xchg + kXBytes;
+  char* const ds_xchg = p_xchg;  // dS^T overwrites P^T in place (same lane, same address)
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
