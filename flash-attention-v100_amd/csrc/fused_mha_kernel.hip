@@ -110,13 +110,21 @@ __device__ __forceinline__ float add_halves(h8 x, float acc) {
 // Work-group id -> (batch*head slice, block inside the slice).  Consecutive
 // work-group ids go round-robin over the 8 XCDs, each with a private L2; the
 // remap hands every XCD whole (batch, head) slices, so the blocks that stream
-// the same K/V (or Q/dO) rows share one L2.
+// the same K/V (or Q/dO) rows share one L2.  Inside an XCD the blocks are
+// ordered block-index major over its slices: callers number blocks heaviest
+// first, so under causal masking all heavy blocks start before any light one
+// (longest-processing-time-first), which keeps the tail of the launch short.
 __device__ __forceinline__ void slice_and_block(int blocks_per_slice, int& slice, int& blk) {
   const int lin = blockIdx.x, total = gridDim.x;
-  int virt = lin;
-  if ((total & 7) == 0) virt = (lin & 7) * (total >> 3) + (lin >> 3);
-  slice = virt / blocks_per_slice;
-  blk = virt - slice * blocks_per_slice;
+  const int slices = total / blocks_per_slice;
+  if ((slices & 7) == 0) {
+    const int xcd = lin & 7, slot = lin >> 3, spx = slices >> 3;  // slices per XCD
+    blk = slot / spx;
+    slice = xcd * spx + (slot - blk * spx);
+  } else {
+    slice = lin / blocks_per_slice;
+    blk = lin - slice * blocks_per_slice;
+  }
 }
 
 // ---------------------------------------------------------------------------
