@@ -608,6 +608,27 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
 
+  // P^T = exp2(S^T*c - lse2) -> LDS.  MASKED tiles straddle the diagonal or the
+  // end of the sequence.
+  auto probabilities = [&](const f16v (&x)[2], int key0, auto masked_tag) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value != 0;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb) {
+      h8 y0, y1;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float p = fast_exp2(fmaf(x[rb][r], c, -stat));
+        if (MASKED) {
+          const int key = key0 + acc_row(rb, r, hh);
+          if ((CAUSAL && key > qi) || key >= N) p = 0.f;
+        }
+        if (r < 8) y0[r] = (half_t)p; else y1[r - 8] = (half_t)p;
+      }
+      *reinterpret_cast<h8*>(p_mine + rb * 2048) = y0;
+      *reinterpret_cast<h8*>(p_mine + rb * 2048 + 16) = y1;
+    }
+  };
+
   wait_vm<0>();  // resident rows, statistics and the first copies
   int s0 = 0, s2 = 2;  // j % 3, (j + 2) % 3
   for (int j = 0; j < nt; ++j) {
@@ -644,21 +665,8 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
         __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
       }
       if (!role_b) {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-          h8 y0, y1;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            float p = fast_exp2(fmaf(x[rb][r], c, -stat));
-            if (masked) {
-              const int key = key0 + acc_row(rb, r, hh);
-              if ((CAUSAL && key > qi) || key >= N) p = 0.f;
-            }
-            if (r < 8) y0[r] = (half_t)p; else y1[r - 8] = (half_t)p;
-          }
-          *reinterpret_cast<h8*>(p_mine + rb * 2048) = y0;
-          *reinterpret_cast<h8*>(p_mine + rb * 2048 + 16) = y1;
-        }
+        if (masked) probabilities(x, key0, IntTag<1>{});
+        else probabilities(x, key0, IntTag<0>{});
       } else {
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
@@ -880,6 +888,28 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
 
+  // P = exp2(S*c - lse2), fp16, in B-operand order.  MASKED tiles straddle the
+  // diagonal or the end of the sequence.
+  auto probabilities = [&](const f16v (&x)[2], h8 (&y)[4], const char* Sl, int q0, auto masked_tag)
+                           __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_tag)::value != 0;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f4v l4 = *reinterpret_cast<const f4v*>(Sl + (rb * 32 + 8 * g) * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float p = fast_exp2(fmaf(x[rb][4 * g + e], c, -l4[e]));
+          if (MASKED) {
+            const int q = q0 + rb * 32 + 8 * g + 4 * hh + e;
+            if ((CAUSAL && ki > q) || q >= N) p = 0.f;
+          }
+          y[rb * 2 + (g >> 1)][(g & 1) * 4 + e] = (half_t)p;
+        }
+      }
+  };
+
   wait_vm<0>();  // resident rows and the first copies: nothing is left for the compiler to wait on in the loop
   int s0 = 0, s2 = 2;  // it % 3, (it + 2) % 3
   for (int it = 0; it < n_it; ++it) {
@@ -903,21 +933,8 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     if (active) {
       if (!role_b) {
         gemm1(Ql, x);
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const f4v l4 = *reinterpret_cast<const f4v*>(Sl + (rb * 32 + 8 * g) * 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              float p = fast_exp2(fmaf(x[rb][4 * g + e], c, -l4[e]));
-              if (masked) {
-                const int q = q0 + rb * 32 + 8 * g + 4 * hh + e;
-                if ((CAUSAL && ki > q) || q >= N) p = 0.f;
-              }
-              y[rb * 2 + (g >> 1)][(g & 1) * 4 + e] = (half_t)p;
-            }
-          }
+        if (masked) probabilities(x, y, Sl, q0, IntTag<1>{});
+        else probabilities(x, y, Sl, q0, IntTag<0>{});
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
           *reinterpret_cast<h8*>(p_mine + rb * 2048) = y[rb * 2];
