@@ -728,15 +728,17 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 // Backward, dK/dV pass.  Block = 128 keys = 4 pairs of waves; a pair owns 32
 // keys and splits the work so that each wave keeps only one accumulator and one
 // of K / V in registers (two waves per SIMD fit):
-//   wave A (waves 0-3): S = Q K^T, P = exp(S - lse)   -> P to LDS,  dV^T += dO^T P
-//   wave B (waves 4-7): dP = dO V^T, T = dP - delta   <- P from LDS, dS = P o T,
-//                                                      dK^T += Q^T dS
+//   wave A (waves 0-3), tile j:   S = Q K^T, P = exp(S - lse) -> P(j) to LDS,
+//                                 dV^T += dO^T P
+//   wave B (waves 4-7), tile j:   dS(j-1) = P(j-1) o T(j-1),  dK^T += Q(j-1)^T dS(j-1),
+//                                 then dP = dO(j) V^T, T(j) = dP - delta (kept in registers)
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 618-629, 653-656,
-// 697-712; key-block-parallel launch as at :908-915).  P travels in the
-// accumulator layout, lane for lane, so no transposition is involved.  Q/dO
-// tiles of 64 queries stream through a 3-slot LDS ring, copied two tiles
-// ahead, with the tile's lse2 and delta rows.  Two barriers per tile: one for
-// the tile, one for P.
+// 697-712; key-block-parallel launch as at :908-915).  B runs one tile behind A
+// for the part that needs P, so one barrier per tile is enough and neither wave
+// waits for the other inside a tile.  P travels in the accumulator layout, lane
+// for lane (double-buffered).  Q tiles of 64 queries stream through a 4-slot
+// LDS ring (B still needs tile j-1), dO tiles and the tile's lse2/delta rows
+// through 3-slot rings, all copied two tiles ahead.
 // ---------------------------------------------------------------------------
 constexpr int kKvPairs = 4;
 constexpr int kKvWaves = 2 * kKvPairs;
@@ -751,14 +753,14 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kKvWaves;  // copies per wave per tile, per tensor
-  // Q ring, dO ring, per slot 64 lse2 then 64 delta values (1 KiB, half unused),
-  // and the P exchange: per pair two 32x32 fp16 blocks, 32 bytes per lane each.
+  // Q ring (4), dO ring (3), per stats slot 64 lse2 then 64 delta values (1 KiB, half
+  // unused), and the P exchange: 2 buffers x per pair two 32x32 fp16 blocks (32 bytes per lane each).
   constexpr int kStBytes = 1024;
   constexpr int kPBytes = kKvPairs * 2 * 2048;
-  __shared__ __attribute__((aligned(1024))) char smem[3 * (2 * T::kBytes + kStBytes) + kPBytes];
+  __shared__ __attribute__((aligned(1024))) char smem[7 * T::kBytes + 3 * kStBytes + 2 * kPBytes];
   char* const q_ring = smem;
-  char* const g_ring = smem + 3 * T::kBytes;
-  char* const st_ring = smem + 6 * T::kBytes;
+  char* const g_ring = smem + 4 * T::kBytes;
+  char* const st_ring = smem + 7 * T::kBytes;
   char* const p_xchg = st_ring + 3 * kStBytes;
 
   const int lane = threadIdx.x & 63;
@@ -797,12 +799,12 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   // 16-31 its 64 delta values, 4 floats each; lanes 32-63 repeat them into unused space.
   const int st_quad = (lane & 15) * 4;
   const bool st_is_delta = (lane >> 4) & 1;
-  auto copy_tiles = [&](int slot, int tile_idx) __attribute__((always_inline)) {
-    const int row0 = tile_idx * kTile;
+  auto copy_tiles = [&](int it) __attribute__((always_inline)) {  // tile t_begin + it
+    const int row0 = (t_begin + it) * kTile;
     const half_t* qp = Qb + (long)row0 * rs;   // wave-uniform
     const half_t* gp = dOb + (long)row0 * rs;
-    char* qdst = q_ring + slot * T::kBytes;
-    char* gdst = g_ring + slot * T::kBytes;
+    char* qdst = q_ring + (it & 3) * T::kBytes;
+    char* gdst = g_ring + (it % 3) * T::kBytes;
     if (row0 + kTile <= N) {
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) copy16(qp, c_goff[u], qdst + c_blk[u]);
@@ -824,12 +826,12 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
       // N is a multiple of 32, so a quad of rows is either inside or outside [0, N)
       const int quad = min(row0 + st_quad, N - 4);
       copy16(reinterpret_cast<const half_t*>(delta_b), quad * 4 + (st_is_delta ? 0 : lse2_off),
-             st_ring + slot * kStBytes);
+             st_ring + (it % 3) * kStBytes);
     }
   };
 
-  copy_tiles(0, t_begin);
-  if (n_it > 1) copy_tiles(1, t_begin + 1);
+  copy_tiles(0);
+  if (n_it > 1) copy_tiles(1);
 
   // resident rows of this wave: K for role A, V for role B
   h8 rf[G::kKSteps];
@@ -843,7 +845,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   swz_rows_off<D>(lane, r_off);
   swz_cols_off<D>(lane, c_off);
   const int st_off = hh * 16 + (role_b ? 256 : 0);   // + (rb * 32 + 8 * g) * 4: this role's quad
-  char* const p_mine = p_xchg + pair * 4096 + lane * 32;  // + rb * 2048
+  char* const p_mine = p_xchg + pair * 4096 + lane * 32;  // + buffer * kPBytes + rb * 2048
 
   f16v acc[G::kDBlocks];  // dV^T (role A) or dK^T (role B)
 #pragma unroll
@@ -887,7 +889,6 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     }
     __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
-
   // P = exp2(S*c - lse2), fp16, in B-operand order.  MASKED tiles straddle the
   // diagonal or the end of the sequence.
   auto probabilities = [&](const f16v (&x)[2], h8 (&y)[4], const char* Sl, int q0, auto masked_tag)
@@ -909,11 +910,13 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
         }
       }
   };
+  auto tile_active = [&](int it) __attribute__((always_inline)) {
+    return !CAUSAL || (t_begin + it) * kTile + kTile - 1 >= k0w;
+  };
 
-  wait_vm<0>();  // resident rows and the first copies: nothing is left for the compiler to wait on in the loop
-  int s0 = 0, s2 = 2;  // it % 3, (it + 2) % 3
-  for (int it = 0; it < n_it; ++it) {
-    // tile `it` was issued two iterations ago; the copies of tile it+1 may still be in flight
+  // Per iteration: wait for tile `it` (issued two iterations ago; the copies of tile
+  // it+1 may still be in flight), one barrier, issue the copies of tile it+2.
+  auto step_sync = [&](int it) __attribute__((always_inline)) {
     if (it + 1 < n_it) {
       if (wave == 0) wait_vm<2 * kIPW + 1>();
       else wait_vm<2 * kIPW>();
@@ -921,26 +924,59 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
       wait_vm<0>();
     }
     block_barrier();
-    if (it + 2 < n_it) copy_tiles(s2, t_begin + it + 2);
-    const char* Ql = q_ring + s0 * T::kBytes;
-    const char* Gl = g_ring + s0 * T::kBytes;
-    const char* Sl = st_ring + s0 * kStBytes + st_off;
-    const int q0 = (t_begin + it) * kTile;
-    const bool active = !CAUSAL || q0 + kTile - 1 >= k0w;
-    const bool masked = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
-    h8 y[4];      // role A: P, role B: dS, fp16 in B-operand order
-    f16v x[2];    // role A: S, role B: dP - delta
-    if (active) {
-      if (!role_b) {
+    if (it + 2 < n_it) copy_tiles(it + 2);
+  };
+  wait_vm<0>();  // resident rows and the first copies: nothing is left for the compiler to wait on in the loops
+  if (!role_b) {
+    for (int it = 0; it <= n_it; ++it) {
+      step_sync(it);
+      if (it < n_it && tile_active(it)) {
+        const char* Ql = q_ring + (it & 3) * T::kBytes;
+        const char* Gl = g_ring + (it % 3) * T::kBytes;
+        const char* Sl = st_ring + (it % 3) * kStBytes + st_off;
+        const int q0 = (t_begin + it) * kTile;
+        const bool masked = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
+        f16v x[2];
+        h8 y[4];
         gemm1(Ql, x);
         if (masked) probabilities(x, y, Sl, q0, IntTag<1>{});
         else probabilities(x, y, Sl, q0, IntTag<0>{});
+        char* pw = p_mine + (it & 1) * kPBytes;
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
-          *reinterpret_cast<h8*>(p_mine + rb * 2048) = y[rb * 2];
-          *reinterpret_cast<h8*>(p_mine + rb * 2048 + 16) = y[rb * 2 + 1];
+          *reinterpret_cast<h8*>(pw + rb * 2048) = y[rb * 2];
+          *reinterpret_cast<h8*>(pw + rb * 2048 + 16) = y[rb * 2 + 1];
         }
-      } else {
+        gemm2(Gl, y);
+      }
+    }
+  } else {
+    f16v x[2];  // dP - delta of the previous tile
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
+    for (int it = 0; it <= n_it; ++it) {
+      step_sync(it);
+      if (it >= 1 && tile_active(it - 1)) {  // the part that needs P, one tile behind
+        const char* Ql = q_ring + ((it - 1) & 3) * T::kBytes;
+        const char* pr = p_mine + ((it - 1) & 1) * kPBytes;
+        h8 y[4];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+          const h8 p0 = *reinterpret_cast<const h8*>(pr + rb * 2048);
+          const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 16);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
+            y[rb * 2 + 1][e] = (half_t)((float)p1[e] * x[rb][8 + e]);
+          }
+        }
+        gemm2(Ql, y);
+      }
+      if (it < n_it && tile_active(it)) {
+        const char* Gl = g_ring + (it % 3) * T::kBytes;
+        const char* Sl = st_ring + (it % 3) * kStBytes + st_off;
         gemm1(Gl, x);
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
@@ -952,26 +988,6 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
           }
       }
     }
-    block_barrier();  // P of this tile is in LDS
-    if (active) {
-      if (!role_b) {
-        gemm2(Gl, y);
-      } else {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-          const h8 p0 = *reinterpret_cast<const h8*>(p_mine + rb * 2048);
-          const h8 p1 = *reinterpret_cast<const h8*>(p_mine + rb * 2048 + 16);
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
-            y[rb * 2 + 1][e] = (half_t)((float)p1[e] * x[rb][8 + e]);
-          }
-        }
-        gemm2(Ql, y);
-      }
-    }
-    s2 = s0;
-    s0 = s0 == 2 ? 0 : s0 + 1;
   }
 
   if (!role_b) store_resident<D>(dV + head_off, rs, ki, N, acc, 1.f, hh);
