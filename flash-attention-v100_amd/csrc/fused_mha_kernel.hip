@@ -491,15 +491,16 @@ fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ d
 // ---------------------------------------------------------------------------
 // Backward, dQ pass.  Block = 128 queries = 4 pairs of waves; a pair owns 32
 // queries and splits the work (two waves per SIMD fit):
-//   wave A (waves 0-3): S^T = K Q^T, P^T = exp(S^T - lse)   -> P^T to LDS
-//   wave B (waves 4-7): dP^T = V dO^T, T = dP^T - delta      <- P^T from LDS,
-//                       dS^T = P^T o T                       -> dS^T to LDS
-//   both:               dQ^T += K^T dS^T, each for half of the head dimension
+//   wave A (waves 0-3), tile j: S^T = K Q^T, P^T = exp(S^T - lse) -> P^T(j) to LDS
+//   wave B (waves 4-7), tile j: dS^T(j-1) = P^T(j-1) o T(j-1), dQ^T += K(j-1)^T dS^T(j-1),
+//                               then dP^T = V(j) dO^T, T(j) = dP^T - delta (kept in registers)
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 653-656, 680-683).
-// lse and delta belong to the resident query, so they are per-lane scalars.
-// P^T and dS^T travel in the accumulator layout, lane for lane.  K/V tiles of 64
-// keys stream through a 3-slot LDS ring, copied two tiles ahead.  Three barriers
-// per tile: the tile, P^T, dS^T.
+// B runs one tile behind A for the part that needs P^T, so one barrier per tile
+// is enough and neither wave waits for the other inside a tile.  lse and delta
+// belong to the resident query, so they are per-lane scalars.  P^T travels in
+// the accumulator layout, lane for lane (double-buffered).  K tiles of 64 keys
+// stream through a 4-slot LDS ring (B still needs tile j-1), V tiles through a
+// 3-slot ring, both copied two tiles ahead.
 // ---------------------------------------------------------------------------
 constexpr int kDqPairs = 4;
 constexpr int kDqWaves = 2 * kDqPairs;
@@ -514,14 +515,12 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kDqWaves;  // copies per wave per tile, per tensor
-  constexpr int kHalfDB = G::kDBlocks / 2;     // 32-feature blocks of dQ per wave
-  // K ring, V ring, then per pair a 64x32 fp16 block (4 KiB) holding P^T and later dS^T
-  constexpr int kXBytes = kDqPairs * 4096;
-  __shared__ __attribute__((aligned(1024))) char smem[2 * 3 * T::kBytes + kXBytes];
+  // K ring (4), V ring (3), then two buffers of per pair a 64x32 fp16 block (4 KiB) of P^T
+  constexpr int kPBytes = kDqPairs * 4096;
+  __shared__ __attribute__((aligned(1024))) char smem[7 * T::kBytes + 2 * kPBytes];
   char* const k_ring = smem;
-  char* const v_ring = smem + 3 * T::kBytes;
-  char* const p_xchg = smem + 6 * T::kBytes;
-  char* const ds_xchg = p_xchg;  // dS^T overwrites P^T in place (same lane, same address)
+  char* const v_ring = smem + 4 * T::kBytes;
+  char* const p_xchg = smem + 7 * T::kBytes;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -542,8 +541,8 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   const int qi = q0w + i;
   const int qrow = min(qi, N - 1);
 
-  int nt = (N + kTile - 1) / kTile;
-  int ntw = nt;
+  int nt = (N + kTile - 1) / kTile;  // tiles the block streams
+  int ntw = nt;                      // tiles this pair takes part in
   if (CAUSAL) {
     nt = min(nt, (min(m0 + kDqBlockQ, N) - 1) / kTile + 1);
     ntw = min(nt, (min(q0w + kResident, N) - 1) / kTile + 1);
@@ -557,12 +556,12 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
     copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
     c_blk[u] = t * 1024;
   }
-  auto copy_tiles = [&](int slot, int tile_idx) __attribute__((always_inline)) {
-    const int row0 = tile_idx * kTile;
+  auto copy_tiles = [&](int j) __attribute__((always_inline)) {
+    const int row0 = j * kTile;
     const half_t* kp = Kb + (long)row0 * rs;  // wave-uniform
     const half_t* vp = Vb + (long)row0 * rs;
-    char* kdst = k_ring + slot * T::kBytes;
-    char* vdst = v_ring + slot * T::kBytes;
+    char* kdst = k_ring + (j & 3) * T::kBytes;
+    char* vdst = v_ring + (j % 3) * T::kBytes;
     if (row0 + kTile <= N) {
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) copy16(kp, c_goff[u], kdst + c_blk[u]);
@@ -582,8 +581,8 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
     }
   };
 
-  copy_tiles(0, 0);
-  if (nt > 1) copy_tiles(1, 1);
+  copy_tiles(0);
+  if (nt > 1) copy_tiles(1);
 
   // resident rows of this wave: Q for role A, dO for role B; and the row statistic it needs
   h8 rf[G::kKSteps];
@@ -598,19 +597,31 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   int r_off[2], c_off[2];
   swz_rows_off<D>(lane, r_off);
   swz_cols_off<D>(lane, c_off);
-  char* const p_mine = p_xchg + pair * 4096 + lane * 32;    // + rb * 2048
-  char* const ds_mine = ds_xchg + pair * 4096 + lane * 32;  // + rb * 2048
-  const int db0 = role_b ? kHalfDB : 0;  // first 32-feature block of dQ this wave accumulates
+  char* const p_mine = p_xchg + pair * 4096 + lane * 32;  // + buffer * kPBytes + rb * 2048
 
-  f16v dq[kHalfDB];
+  // first GEMM of a tile: rows of K (role A) or V (role B) against the resident rows
+  auto gemm1 = [&](const char* tile_lds, f16v (&x)[2]) __attribute__((always_inline)) {
 #pragma unroll
-  for (int db = 0; db < kHalfDB; ++db)
+    for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
-
+      for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) x[rb] = mfma(swz_rows<D>(tile_lds, rb, kk, r_off), rf[kk], x[rb]);
+    }
+    constexpr int kN = 2 * G::kKSteps, kLead = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
+#pragma unroll
+    for (int n = 0; n < kN - kLead; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
+  };
   // P^T = exp2(S^T*c - lse2) -> LDS.  MASKED tiles straddle the diagonal or the
   // end of the sequence.
-  auto probabilities = [&](const f16v (&x)[2], int key0, auto masked_tag) __attribute__((always_inline)) {
+  auto probabilities = [&](const f16v (&x)[2], char* pw, int key0, auto masked_tag) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_tag)::value != 0;
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb) {
@@ -624,103 +635,83 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
         }
         if (r < 8) y0[r] = (half_t)p; else y1[r - 8] = (half_t)p;
       }
-      *reinterpret_cast<h8*>(p_mine + rb * 2048) = y0;
-      *reinterpret_cast<h8*>(p_mine + rb * 2048 + 16) = y1;
+      *reinterpret_cast<h8*>(pw + rb * 2048) = y0;
+      *reinterpret_cast<h8*>(pw + rb * 2048 + 16) = y1;
     }
   };
-
-  wait_vm<0>();  // resident rows, statistics and the first copies
-  int s0 = 0, s2 = 2;  // j % 3, (j + 2) % 3
-  for (int j = 0; j < nt; ++j) {
-    // tile j was issued two iterations ago; the copies of tile j+1 may still be in flight
+  // Per iteration: wait for tile j (issued two iterations ago; the copies of tile
+  // j+1 may still be in flight), one barrier, issue the copies of tile j+2.
+  auto step_sync = [&](int j) __attribute__((always_inline)) {
     if (j + 1 < nt) wait_vm<2 * kIPW>();
     else wait_vm<0>();
     block_barrier();
-    if (j + 2 < nt) copy_tiles(s2, j + 2);
-    const char* Kl = k_ring + s0 * T::kBytes;
-    const char* Vl = v_ring + s0 * T::kBytes;
-    const bool active = j < ntw;
-    const int key0 = j * kTile;
-    const bool masked = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
-    f16v x[2];  // role A: S^T, role B: dP^T - delta
-    if (active) {
-      const char* tl = role_b ? Vl : Kl;
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < G::kKSteps; ++kk) {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) x[rb] = mfma(swz_rows<D>(tl, rb, kk, r_off), rf[kk], x[rb]);
+    if (j + 2 < nt) copy_tiles(j + 2);
+  };
+
+  wait_vm<0>();  // resident rows, statistics and the first copies
+  if (!role_b) {
+    for (int j = 0; j <= nt; ++j) {
+      step_sync(j);
+      if (j < ntw) {
+        const int key0 = j * kTile;
+        const bool masked = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
+        f16v x[2];
+        gemm1(k_ring + (j & 3) * T::kBytes, x);
+        char* pw = p_mine + (j & 1) * kPBytes;
+        if (masked) probabilities(x, pw, key0, IntTag<1>{});
+        else probabilities(x, pw, key0, IntTag<0>{});
       }
-      {
-        constexpr int kN = 2 * G::kKSteps, kLead = 4;
-        __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
+    }
+  } else {
+    f16v dq[G::kDBlocks];
+#pragma unroll
+    for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
+    f16v x[2];  // dP^T - delta of the previous tile
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
+    for (int j = 0; j <= nt; ++j) {
+      step_sync(j);
+      if (j >= 1 && j - 1 < ntw) {  // the part that needs P^T, one tile behind
+        const char* Kl = k_ring + ((j - 1) & 3) * T::kBytes;
+        const char* pr = p_mine + ((j - 1) & 1) * kPBytes;
+        h8 y[4];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+          const h8 p0 = *reinterpret_cast<const h8*>(pr + rb * 2048);
+          const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 16);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
+            y[rb * 2 + 1][e] = (half_t)((float)p1[e] * x[rb][8 + e]);
+          }
+        }
+#pragma unroll
+        for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+          for (int db = 0; db < G::kDBlocks; ++db) dq[db] = mfma(swz_cols<D>(Kl, c16, db, c_off), y[c16], dq[db]);
+        }
+        constexpr int kN = 4 * G::kDBlocks, kLead = 4;
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead, 0);
 #pragma unroll
         for (int n = 0; n < kN - kLead; ++n) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
       }
-      if (!role_b) {
-        if (masked) probabilities(x, key0, IntTag<1>{});
-        else probabilities(x, key0, IntTag<0>{});
-      } else {
+      if (j < ntw) {
+        gemm1(v_ring + (j % 3) * T::kBytes, x);
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) x[rb][r] -= stat;
       }
     }
-    block_barrier();  // P^T of this tile is in LDS
-    if (active && role_b) {
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-        const h8 p0 = *reinterpret_cast<const h8*>(p_mine + rb * 2048);
-        const h8 p1 = *reinterpret_cast<const h8*>(p_mine + rb * 2048 + 16);
-        h8 y0, y1;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          y0[e] = (half_t)((float)p0[e] * x[rb][e]);
-          y1[e] = (half_t)((float)p1[e] * x[rb][8 + e]);
-        }
-        *reinterpret_cast<h8*>(ds_mine + rb * 2048) = y0;
-        *reinterpret_cast<h8*>(ds_mine + rb * 2048 + 16) = y1;
-      }
-    }
-    block_barrier();  // dS^T of this tile is in LDS
-    if (active) {
-      h8 y[4];
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-        y[rb * 2] = *reinterpret_cast<const h8*>(ds_mine + rb * 2048);
-        y[rb * 2 + 1] = *reinterpret_cast<const h8*>(ds_mine + rb * 2048 + 16);
-      }
-#pragma unroll
-      for (int c16 = 0; c16 < 4; ++c16) {
-#pragma unroll
-        for (int db = 0; db < kHalfDB; ++db) dq[db] = mfma(swz_cols<D>(Kl, c16, db0 + db, c_off), y[c16], dq[db]);
-      }
-    }
-    s2 = s0;
-    s0 = s0 == 2 ? 0 : s0 + 1;
-  }
-
-  // each wave of the pair stores its half of the head dimension
-  if (qi < N) {
-    half_t* op = dQ + head_off + (long)qi * rs + db0 * 32;
-#pragma unroll
-    for (int db = 0; db < kHalfDB; ++db) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        h4 v;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = (half_t)(dq[db][4 * g + e] * scale);
-        *reinterpret_cast<h4*>(op + db * 32 + 8 * g + 4 * hh) = v;
-      }
-    }
+    store_resident<D>(dQ + head_off, rs, qi, N, dq, scale, hh);
   }
 }
 
