@@ -96,17 +96,6 @@ __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long r
   }
 }
 
-// Sum of the 8 halves of x added to acc, two at a time (v_dot2_f32_f16).
-__device__ __forceinline__ float add_halves(h8 x, float acc) {
-  const h2 ones = {(half_t)1.f, (half_t)1.f};
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    h2 pr = {x[2 * j], x[2 * j + 1]};
-    acc = __builtin_amdgcn_fdot2(pr, ones, acc, false);
-  }
-  return acc;
-}
-
 // Work-group id -> (batch*head slice, block inside the slice).  Consecutive
 // work-group ids go round-robin over the 8 XCDs, each with a private L2; the
 // remap hands every XCD whole (batch, head) slices, so the blocks that stream
@@ -384,13 +373,23 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
     }
+    // Row sums with plain fp32 adds: the dot-product instructions share the
+    // matrix pipeline and stall behind the other wave's MFMAs.
     const float mc = m_run * c;
+    float l0 = 0.f, l1 = 0.f;
 #pragma unroll
     for (int c16 = 0; c16 < 4; ++c16) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) pf[c16][e] = (half_t)fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + e], c, -mc));
-      l_run = add_halves(pf[c16], l_run);
+      for (int e = 0; e < 8; e += 2) {
+        const float p0 = fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + e], c, -mc));
+        const float p1 = fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + e + 1], c, -mc));
+        pf[c16][e] = (half_t)p0;
+        pf[c16][e + 1] = (half_t)p1;
+        l0 += p0;
+        l1 += p1;
+      }
     }
+    l_run += l0 + l1;
   };
   auto accumulate = [&](const char* Vl, int t) __attribute__((always_inline)) {
     if (t < 0 || t >= ntw) return;
