@@ -596,7 +596,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   int r_off[2], c_off[2];
   swz_rows_off<D>(lane, r_off);
   swz_cols_off<D>(lane, c_off);
-  char* const p_mine = p_xchg + pair * 4096 + lane * 32;  // + buffer * kPBytes + rb * 2048
+  char* const p_mine = p_xchg + pair * 4096 + lane * 16;  // + buffer * kPBytes + rb * 2048 + half * 1024
 
   // first GEMM of a tile: rows of K (role A) or V (role B) against the resident rows
   auto gemm1 = [&](const char* tile_lds, f16v (&x)[2]) __attribute__((always_inline)) {
@@ -635,7 +635,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
         if (r < 8) y0[r] = (half_t)p; else y1[r - 8] = (half_t)p;
       }
       *reinterpret_cast<h8*>(pw + rb * 2048) = y0;
-      *reinterpret_cast<h8*>(pw + rb * 2048 + 16) = y1;
+      *reinterpret_cast<h8*>(pw + rb * 2048 + 1024) = y1;
     }
   };
   // Per iteration: wait for tile j (issued two iterations ago; the copies of tile
@@ -681,7 +681,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
           const h8 p0 = *reinterpret_cast<const h8*>(pr + rb * 2048);
-          const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 16);
+          const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 1024);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
@@ -744,7 +744,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kKvWaves;  // copies per wave per tile, per tensor
   // Q ring (4), dO ring (3), per stats slot 64 lse2 then 64 delta values (1 KiB, half
-  // unused), and the P exchange: 2 buffers x per pair two 32x32 fp16 blocks (32 bytes per lane each).
+  // unused), and the P exchange: 2 buffers x per pair two 32x32 fp16 blocks (two 16-byte halves per lane each, in separate 1 KiB planes so that the 16-byte accesses are free of bank conflicts).
   constexpr int kStBytes = 1024;
   constexpr int kPBytes = kKvPairs * 2 * 2048;
   __shared__ __attribute__((aligned(1024))) char smem[7 * T::kBytes + 3 * kStBytes + 2 * kPBytes];
@@ -835,7 +835,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   swz_rows_off<D>(lane, r_off);
   swz_cols_off<D>(lane, c_off);
   const int st_off = hh * 16 + (role_b ? 256 : 0);   // + (rb * 32 + 8 * g) * 4: this role's quad
-  char* const p_mine = p_xchg + pair * 4096 + lane * 32;  // + buffer * kPBytes + rb * 2048
+  char* const p_mine = p_xchg + pair * 4096 + lane * 16;  // + buffer * kPBytes + rb * 2048 + half * 1024
 
   f16v acc[G::kDBlocks];  // dV^T (role A) or dK^T (role B)
 #pragma unroll
@@ -935,7 +935,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
           *reinterpret_cast<h8*>(pw + rb * 2048) = y[rb * 2];
-          *reinterpret_cast<h8*>(pw + rb * 2048 + 16) = y[rb * 2 + 1];
+          *reinterpret_cast<h8*>(pw + rb * 2048 + 1024) = y[rb * 2 + 1];
         }
         gemm2(Gl, y);
       }
@@ -955,7 +955,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
           const h8 p0 = *reinterpret_cast<const h8*>(pr + rb * 2048);
-          const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 16);
+          const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 1024);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
