@@ -492,7 +492,8 @@ fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ d
 // queries and splits the work (two waves per SIMD fit):
 //   wave A (waves 0-3), tile j: S^T = K Q^T, P^T = exp(S^T - lse) -> P^T(j) to LDS
 //   wave B (waves 4-7), tile j: dS^T(j-1) = P^T(j-1) o T(j-1), dQ^T += K(j-1)^T dS^T(j-1),
-//                               then dP^T = V(j) dO^T, T(j) = dP^T - delta (kept in registers)
+//                               then dP^T = V(j) dO^T, T(j) = dP^T - delta (kept in registers,
+//                               as -T: the GEMM runs on -dO with accumulators that start at delta)
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 653-656, 680-683).
 // B runs one tile behind A for the part that needs P^T, so one barrier per tile
 // is enough and neither wave waits for the other inside a tile.  lse and delta
@@ -588,7 +589,12 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   {
     const half_t* rp = (role_b ? dO : Q) + head_off + (long)qrow * rs + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+      rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
+      // Role B works with -dO: its first GEMM then gives delta - dP^T on top of
+      // accumulators that start at delta, with no subtraction afterwards.
+      if (role_b) rf[kk] = -rf[kk];
+    }
   }
   const long stat_at = ((long)b * H + h) * N + qrow;
   const float stat = role_b ? delta[stat_at] : LSE[stat_at] * kLog2e;
@@ -598,12 +604,13 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   swz_cols_off<D>(lane, c_off);
   char* const p_mine = p_xchg + pair * 4096 + lane * 16;  // + buffer * kPBytes + rb * 2048 + half * 1024
 
-  // first GEMM of a tile: rows of K (role A) or V (role B) against the resident rows
-  auto gemm1 = [&](const char* tile_lds, f16v (&x)[2]) __attribute__((always_inline)) {
+  // first GEMM of a tile: rows of K (role A) or V (role B) against the resident
+  // rows, on top of the value `init` in every accumulator element
+  auto gemm1 = [&](const char* tile_lds, f16v (&x)[2], float init) __attribute__((always_inline)) {
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
+      for (int r = 0; r < 16; ++r) x[rb][r] = init;
 #pragma unroll
     for (int kk = 0; kk < G::kKSteps; ++kk) {
 #pragma unroll
@@ -655,7 +662,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
         const int key0 = j * kTile;
         const bool masked = (CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N);
         f16v x[2];
-        gemm1(k_ring + (j & 3) * T::kBytes, x);
+        gemm1(k_ring + (j & 3) * T::kBytes, x, 0.f);
         char* pw = p_mine + (j & 1) * kPBytes;
         if (masked) probabilities(x, pw, key0, IntTag<1>{});
         else probabilities(x, pw, key0, IntTag<0>{});
@@ -667,7 +674,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
     for (int db = 0; db < G::kDBlocks; ++db)
 #pragma unroll
       for (int r = 0; r < 16; ++r) dq[db][r] = 0.f;
-    f16v x[2];  // dP^T - delta of the previous tile
+    f16v x[2];  // delta - dP^T of the previous tile
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
@@ -684,8 +691,8 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
           const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 1024);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
-            y[rb * 2 + 1][e] = (half_t)((float)p1[e] * x[rb][8 + e]);
+            y[rb * 2][e] = (half_t)(-(float)p0[e] * x[rb][e]);
+            y[rb * 2 + 1][e] = (half_t)(-(float)p1[e] * x[rb][8 + e]);
           }
         }
 #pragma unroll
@@ -702,13 +709,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
         }
         __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
       }
-      if (j < ntw) {
-        gemm1(v_ring + (j % 3) * T::kBytes, x);
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) x[rb][r] -= stat;
-      }
+      if (j < ntw) gemm1(v_ring + (j % 3) * T::kBytes, x, stat);
     }
     store_resident<D>(dQ + head_off, rs, qi, N, dq, scale, hh);
   }
@@ -721,7 +722,8 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 //   wave A (waves 0-3), tile j:   S = Q K^T, P = exp(S - lse) -> P(j) to LDS,
 //                                 dV^T += dO^T P
 //   wave B (waves 4-7), tile j:   dS(j-1) = P(j-1) o T(j-1),  dK^T += Q(j-1)^T dS(j-1),
-//                                 then dP = dO(j) V^T, T(j) = dP - delta (kept in registers)
+//                                 then dP = dO(j) V^T, T(j) = dP - delta (kept in registers, as -T:
+//                                 the GEMM runs on -V with accumulators loaded with delta)
 // (formulas: reference kernel/fused_mha_kernel.cu:598-603, 618-629, 653-656,
 // 697-712; key-block-parallel launch as at :908-915).  B runs one tile behind A
 // for the part that needs P, so one barrier per tile is enough and neither wave
@@ -828,7 +830,12 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   {
     const half_t* rp = (role_b ? V : K) + head_off + (long)krow * rs + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+      rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
+      // Role B works with -V: its first GEMM then gives delta - dP on top of
+      // accumulators loaded with delta, with no subtraction afterwards.
+      if (role_b) rf[kk] = -rf[kk];
+    }
   }
 
   int r_off[2], c_off[2];
@@ -843,12 +850,9 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
 
-  // first GEMM of a tile: rows of Q (role A) or dO (role B) against the resident rows
+  // first GEMM of a tile: rows of Q (role A) or dO (role B) against the resident
+  // rows, on top of what x holds
   auto gemm1 = [&](const char* tile_lds, f16v (&x)[2]) __attribute__((always_inline)) {
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < G::kKSteps; ++kk) {
 #pragma unroll
@@ -928,6 +932,10 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
         const bool masked = (CAUSAL && q0 < k0w + kResident - 1) || (q0 + kTile > N);
         f16v x[2];
         h8 y[4];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
         gemm1(Ql, x);
         if (masked) probabilities(x, y, Sl, q0, IntTag<1>{});
         else probabilities(x, y, Sl, q0, IntTag<0>{});
@@ -941,7 +949,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
       }
     }
   } else {
-    f16v x[2];  // dP - delta of the previous tile
+    f16v x[2];  // delta - dP of the previous tile
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
@@ -958,8 +966,8 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
           const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 1024);
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            y[rb * 2][e] = (half_t)((float)p0[e] * x[rb][e]);
-            y[rb * 2 + 1][e] = (half_t)((float)p1[e] * x[rb][8 + e]);
+            y[rb * 2][e] = (half_t)(-(float)p0[e] * x[rb][e]);
+            y[rb * 2 + 1][e] = (half_t)(-(float)p1[e] * x[rb][8 + e]);
           }
         }
         gemm2(Ql, y);
@@ -967,15 +975,16 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
       if (it < n_it && tile_active(it)) {
         const char* Gl = g_ring + (it % 3) * T::kBytes;
         const char* Sl = st_ring + (it % 3) * kStBytes + st_off;
-        gemm1(Gl, x);
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const f4v d4 = *reinterpret_cast<const f4v*>(Sl + (rb * 32 + 8 * g) * 4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) x[rb][4 * g + e] -= d4[e];
+            for (int e = 0; e < 4; ++e) x[rb][4 * g + e] = d4[e];
           }
+        __builtin_amdgcn_sched_barrier(0);  // keep the delta loads out of the GEMM's read/MFMA pipeline
+        gemm1(Gl, x);
       }
     }
   }
