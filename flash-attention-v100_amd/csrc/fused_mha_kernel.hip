@@ -507,11 +507,17 @@ constexpr int kDqWaves = 2 * kDqPairs;
 constexpr int kDqThreads = kDqWaves * 64;
 constexpr int kDqBlockQ = kDqPairs * kResident;
 
-template <int D, bool CAUSAL>
+// STATS: the kernel also produces the two row statistics of the backward,
+// delta = rowsum(dO o O) and lse2 = lse * log2(e), for its own queries, uses
+// them and stores them in the workspace for the dK/dV pass (which must then be
+// launched after this one); fmha_bwd_delta_kernel is not needed in that case.
+// Otherwise delta is read from the workspace.
+template <int D, bool CAUSAL, bool STATS>
 __global__ void __launch_bounds__(kDqThreads, 1)
 fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-                   const half_t* __restrict__ dO, const float* __restrict__ LSE, const float* __restrict__ delta,
-                   half_t* __restrict__ dQ, int H, int N, int nmb, float c, float scale) {
+                   const half_t* __restrict__ O, const half_t* __restrict__ dO, const float* __restrict__ LSE,
+                   float* __restrict__ delta, float* __restrict__ lse2, half_t* __restrict__ dQ, int H, int N, int nmb,
+                   float c, float scale) {
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kDqWaves;  // copies per wave per tile, per tensor
@@ -586,18 +592,46 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
 
   // resident rows of this wave: Q for role A, dO for role B; and the row statistic it needs
   h8 rf[G::kKSteps];
+  const long stat_at = ((long)b * H + h) * N + qrow;
+  float stat;
   {
     const half_t* rp = (role_b ? dO : Q) + head_off + (long)qrow * rs + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) {
-      rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
-      // Role B works with -dO: its first GEMM then gives delta - dP^T on top of
-      // accumulators that start at delta, with no subtraction afterwards.
-      if (role_b) rf[kk] = -rf[kk];
+    for (int kk = 0; kk < G::kKSteps; ++kk) rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
+    if (STATS) {
+      if (role_b) {
+        // delta of this lane's query.  The lane has every other 8-feature chunk of
+        // the row; the partial sums are combined in the order of
+        // fmha_bwd_delta_kernel's shuffle tree, so both give the same bits.
+        const half_t* op = O + head_off + (long)qrow * rs + hh * 8;
+        float part[G::kKSteps];
+#pragma unroll
+        for (int kk = 0; kk < G::kKSteps; ++kk) {
+          const h8 ov = *reinterpret_cast<const h8*>(op + kk * 16);
+          part[kk] = 0.f;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) part[kk] = fmaf((float)ov[e], (float)rf[kk][e], part[kk]);
+        }
+#pragma unroll
+        for (int stride = G::kKSteps / 2; stride > 0; stride >>= 1)
+#pragma unroll
+          for (int kk = 0; kk < stride; ++kk) part[kk] += part[kk + stride];
+        stat = part[0] + other_half(part[0]);
+        if (hh == 0 && qi < N) delta[stat_at] = stat;
+      } else {
+        stat = LSE[stat_at] * kLog2e;
+        if (hh == 0 && qi < N) lse2[stat_at] = stat;
+      }
+    } else {
+      stat = role_b ? delta[stat_at] : LSE[stat_at] * kLog2e;
+    }
+    // Role B works with -dO: its first GEMM then gives delta - dP^T on top of
+    // accumulators that start at delta, with no subtraction afterwards.
+    if (role_b) {
+#pragma unroll
+      for (int kk = 0; kk < G::kKSteps; ++kk) rf[kk] = -rf[kk];
     }
   }
-  const long stat_at = ((long)b * H + h) * N + qrow;
-  const float stat = role_b ? delta[stat_at] : LSE[stat_at] * kLog2e;
 
   int r_off[2], c_off[2];
   swz_rows_off<D>(lane, r_off);
@@ -1024,7 +1058,9 @@ template <int D, bool CAUSAL>
 int launch_backward(int passes, const void* q, const void* k, const void* v, const void* o, const void* d_o,
                     const void* lse, float* delta, void* dq, void* dk, void* dv, int batch, int head, int n,
                     float scale, hipStream_t stream) {
-  if (passes & kPassDelta) {
+  // With all three passes asked for, the dQ pass produces delta and lse2 itself.
+  const bool dq_makes_stats = (passes & kPassAll) == kPassAll;
+  if ((passes & kPassDelta) && !dq_makes_stats) {
     const long rows = (long)batch * n * head;
     const long threads = rows * (D / 8);
     fmha_bwd_delta_kernel<D><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(
@@ -1034,9 +1070,14 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
   const float c = scale * kLog2e;
   if (passes & kPassDq) {
     const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;
-    fmha_bwd_dq_kernel<D, CAUSAL><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
-        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, (const float*)lse, delta,
-        (half_t*)dq, head, n, nmb, c, scale);
+    if (dq_makes_stats)
+      fmha_bwd_dq_kernel<D, CAUSAL, true><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
+          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o,
+          (const float*)lse, delta, delta + (long)batch * head * n, (half_t*)dq, head, n, nmb, c, scale);
+    else
+      fmha_bwd_dq_kernel<D, CAUSAL, false><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
+          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o,
+          (const float*)lse, delta, delta + (long)batch * head * n, (half_t*)dq, head, n, nmb, c, scale);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   if (passes & kPassDkDv) {
