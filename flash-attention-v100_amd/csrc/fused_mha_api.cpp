@@ -8,8 +8,8 @@
 //   * fwd returns [out, lse] (one logsumexp) instead of [out, max, sum];
 //   * bwd takes lse instead of (D, sum, max); delta is computed on the device
 //     in fp32 inside the launcher;
-//   * head size 64 is accepted as well as 128; seqlen must be a multiple of 32
-//     (the reference assumes it, README.md:3, without checking);
+//   * head size 64 is accepted as well as 128; any seqlen > 0 is accepted (the
+//     reference assumes a multiple of 32, README.md:3, without checking);
 //   * inputs that are not dense (B, N, H, D) are copied dense instead of being
 //     read with wrong strides;
 //   * the arch gate asks for gfx950 instead of sm_70 (:21-23).
@@ -66,7 +66,7 @@ std::vector<at::Tensor> mha_fwd(at::Tensor& q,        // batch x seqlen x heads 
   const int head_size = sizes[3];
   TORCH_CHECK(batch_size > 0, "batch size must be postive");
   TORCH_CHECK(head_size == 64 || head_size == 128, "current repo only supports head dimension 64 or 128");
-  TORCH_CHECK(seqlen_q > 0 && seqlen_q % 32 == 0, "seqlen must be a positive multiple of 32 (right-pad the inputs)");
+  TORCH_CHECK(seqlen_q > 0, "seqlen must be positive");
   CHECK_SHAPE(q, batch_size, seqlen_q, num_heads, head_size);
   CHECK_SHAPE(k, batch_size, seqlen_q, num_heads, head_size);
   CHECK_SHAPE(v, batch_size, seqlen_q, num_heads, head_size);
@@ -121,7 +121,7 @@ std::vector<at::Tensor> mha_bwd(const at::Tensor& dout,  // batch x seqlen x hea
   const int head_size = sizes[3];
   TORCH_CHECK(batch_size > 0, "batch size must be postive");
   TORCH_CHECK(head_size == 64 || head_size == 128, "current repo only supports head dimension 64 or 128");
-  TORCH_CHECK(seqlen_q > 0 && seqlen_q % 32 == 0, "seqlen must be a positive multiple of 32 (right-pad the inputs)");
+  TORCH_CHECK(seqlen_q > 0, "seqlen must be positive");
   CHECK_SHAPE(q, batch_size, seqlen_q, num_heads, head_size);
   CHECK_SHAPE(k, batch_size, seqlen_q, num_heads, head_size);
   CHECK_SHAPE(v, batch_size, seqlen_q, num_heads, head_size);

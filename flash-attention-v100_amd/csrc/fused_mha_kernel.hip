@@ -163,6 +163,19 @@ __device__ __forceinline__ void copy16(const half_t* tile_base, int voff, char* 
       : "memory");
 }
 
+// The same with 4 bytes per lane (256 bytes per instruction): lane l fetches the
+// dword at base + voff and it lands in LDS at lds_dst + 4 * l.
+__device__ __forceinline__ void copy4(const float* base, int voff, char* lds_dst) {
+  const unsigned lds_addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds_dst;
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dword %0, %1"
+      :
+      : "v"(voff), "s"(base), "s"(lds_addr)
+      : "memory");
+}
+
 // rows pattern: lane (i, hh) reads chunk 2*kk + hh of row rb*32 + i.
 // Two lane offsets (kk even / odd); the rest is an immediate.
 template <int D>
@@ -821,10 +834,6 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
     c_blk[u] = t * 1024;
   }
-  // lse2/delta copy (wave 0 only): lanes 0-15 fetch the tile's 64 lse2 values, lanes
-  // 16-31 its 64 delta values, 4 floats each; lanes 32-63 repeat them into unused space.
-  const int st_quad = (lane & 15) * 4;
-  const bool st_is_delta = (lane >> 4) & 1;
   auto copy_tiles = [&](int it) __attribute__((always_inline)) {  // tile t_begin + it
     const int row0 = (t_begin + it) * kTile;
     const half_t* qp = Qb + (long)row0 * rs;   // wave-uniform
@@ -848,11 +857,10 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
         copy16(gp, c_goff[u] - back * rs * 2, gdst + c_blk[u]);
       }
     }
-    if (wave == 0) {
-      // N is a multiple of 32, so a quad of rows is either inside or outside [0, N)
-      const int quad = min(row0 + st_quad, N - 4);
-      copy16(reinterpret_cast<const half_t*>(delta_b), quad * 4 + (st_is_delta ? 0 : lse2_off),
-             st_ring + (it % 3) * kStBytes);
+    if (wave == 0) {  // lane l: lse2 and delta of row row0 + l (rows past the end re-read row N-1)
+      const int at = min(row0 + lane, N - 1) * 4;
+      copy4(delta_b, at + lse2_off, st_ring + (it % 3) * kStBytes);
+      copy4(delta_b, at, st_ring + (it % 3) * kStBytes + 256);
     }
   };
 
@@ -946,7 +954,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   // it+1 may still be in flight), one barrier, issue the copies of tile it+2.
   auto step_sync = [&](int it) __attribute__((always_inline)) {
     if (it + 1 < n_it) {
-      if (wave == 0) wait_vm<2 * kIPW + 1>();
+      if (wave == 0) wait_vm<2 * kIPW + 2>();
       else wait_vm<2 * kIPW>();
     } else {
       wait_vm<0>();
@@ -1031,7 +1039,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 // Host side: validation and launches.
 // ---------------------------------------------------------------------------
 int check_shape(int batch, int head, int m, int n, int d) {
-  if (batch <= 0 || head <= 0 || n <= 0 || m != n || (n % 32) != 0) return FUSED_MHA_ERR_BAD_SHAPE;
+  if (batch <= 0 || head <= 0 || n <= 0 || m != n) return FUSED_MHA_ERR_BAD_SHAPE;
   if (d != 64 && d != 128) return FUSED_MHA_ERR_BAD_HEAD_DIM;
   if ((long)batch * head > 65535) return FUSED_MHA_ERR_TOO_LARGE;
   return FUSED_MHA_OK;
@@ -1175,7 +1183,7 @@ const char* fused_mha_error_string(int code) {
   switch (code) {
     case FUSED_MHA_OK: return "ok";
     case FUSED_MHA_ERR_NULL_POINTER: return "a required pointer is NULL";
-    case FUSED_MHA_ERR_BAD_SHAPE: return "bad shape: need batch, head, n > 0, m == n, n % 32 == 0 and a large enough workspace";
+    case FUSED_MHA_ERR_BAD_SHAPE: return "bad shape: need batch, head, n > 0, m == n and a large enough workspace";
     case FUSED_MHA_ERR_BAD_HEAD_DIM: return "head dimension must be 64 or 128";
     case FUSED_MHA_ERR_MISALIGNED: return "a pointer is not 16-byte aligned";
     case FUSED_MHA_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";

@@ -2,9 +2,10 @@
 flash_attn_v100/flash_attn_interface.py:1-110.
 
 ``flash_attn_func(q, k, v, softmax_scale=None, causal=False)`` takes fp16
-tensors of shape (batch, seqlen, heads, head_size) with seqlen right-padded to a
-multiple of 32 and returns the attention output in the same layout, just like
-the reference.  What differs is behind the extension boundary: the forward
+tensors of shape (batch, seqlen, heads, head_size) and returns the attention
+output in the same layout, just like the reference; seqlen need not be
+right-padded to a multiple of 32 as the reference asks (any length works, a
+padded one still does).  What differs is behind the extension boundary: the forward
 saves one fp32 logsumexp per row instead of separate max and sum tensors, and
 delta = rowsum(dout * out) is computed on the device in fp32 by the backward
 launcher instead of by two fp16 PyTorch ops (reference :43-44).

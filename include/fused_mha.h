@@ -14,7 +14,9 @@
  *     masked score row, i.e. max + ln(sum) of the two statistics the
  *     reference stores separately (kernel/fused_mha_kernel.cu:298-303).
  *   - m == n (self attention, reference: kernel/fused_mha_api.cpp:68-69),
- *     n a multiple of 32 (reference: README.md:3), d is 64 or 128.
+ *     d is 64 or 128.  Any n > 0 is accepted: the last, partial tile is
+ *     handled inside the kernels, so callers need not right-pad the sequence
+ *     to a multiple of 32 as the reference asks (README.md:3).
  *   - causal != 0: key j is visible to query i iff j <= i
  *     (reference: test.py:15-19).
  *   - stream is a hipStream_t passed as void*; NULL is the default stream.
@@ -34,7 +36,7 @@ extern "C" {
 
 #define FUSED_MHA_OK 0
 #define FUSED_MHA_ERR_NULL_POINTER (-1)   /* a required pointer is NULL            */
-#define FUSED_MHA_ERR_BAD_SHAPE (-2)      /* batch/head/n <= 0, m != n, n % 32 != 0 */
+#define FUSED_MHA_ERR_BAD_SHAPE (-2)      /* batch/head/n <= 0, m != n              */
 #define FUSED_MHA_ERR_BAD_HEAD_DIM (-3)   /* d is neither 64 nor 128               */
 #define FUSED_MHA_ERR_MISALIGNED (-4)     /* a pointer is not 16-byte aligned      */
 #define FUSED_MHA_ERR_LAUNCH (-5)         /* the HIP runtime refused the launch    */

@@ -37,7 +37,8 @@ def test_error_strings(lib):
 def test_workspace_bytes(lib):
     assert lib.fused_mha_backward_workspace_bytes(2, 32, 4096, 128) == 2 * 2 * 32 * 4096 * 4
     assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 64) == 2 * 4 * 128 * 4
-    assert lib.fused_mha_backward_workspace_bytes(1, 4, 100, 64) == 0
+    assert lib.fused_mha_backward_workspace_bytes(1, 4, 100, 64) == 2 * 4 * 100 * 4  # any n > 0 is accepted
+    assert lib.fused_mha_backward_workspace_bytes(1, 4, 0, 64) == 0
     assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 96) == 0
 
 
@@ -47,7 +48,7 @@ def test_forward_validation_codes(lib):
     assert f(None, p, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
     assert f(p, p, p, p, None, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
     assert f(p, p, p, p, p, 0, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE
-    assert f(p, p, p, p, p, 1, 1, 48, 48, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE      # n % 32
+    assert f(p, p, p, p, p, 1, 1, 0, 0, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE        # n == 0
     assert f(p, p, p, p, p, 1, 1, 32, 64, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE      # m != n
     assert f(p, p, p, p, p, 1, 1, 32, 32, 96, 1.0, 0, None) == abi.ERR_BAD_HEAD_DIM
     assert f(p, p, p, p, p, 1, 1, 32, 32, 64, float("nan"), 0, None) == abi.ERR_BAD_SCALE
@@ -96,7 +97,7 @@ def test_extension_checks_raise_runtime_error():
         ((ok, t(1, 32, 2, 64, dtype=torch.bfloat16), ok), "same dtype"),
         ((t(32, 2, 64), ok, ok), "4 dimensions"),
         ((t(1, 32, 2, 96), t(1, 32, 2, 96), t(1, 32, 2, 96)), "head dimension"),
-        ((t(1, 48, 2, 64), t(1, 48, 2, 64), t(1, 48, 2, 64)), "multiple of 32"),
+        ((t(1, 0, 2, 64), t(1, 0, 2, 64), t(1, 0, 2, 64)), "seqlen must be positive"),
         ((ok, t(1, 64, 2, 64), ok), "must have shape"),
         ((t(1, 32, 2, 128)[..., ::2], ok, ok), "contiguous last dimension"),
         ((ok, ok, ok), "must be on the GPU"),

@@ -99,6 +99,41 @@ def test_c_abi_small_shapes(lib, B, H, N, D, causal, scale):
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
 
 
+RAGGED = [  # B, H, N, D, causal: lengths that are no multiple of 32 (the last tile is partial)
+    (1, 2, 1, 64, True), (2, 2, 7, 128, False), (1, 3, 33, 64, True), (2, 2, 100, 128, True),
+    (1, 2, 129, 64, False), (1, 2, 257, 128, True), (1, 1, 1000, 128, False), (1, 2, 1031, 64, True),
+]
+
+
+@pytest.mark.parametrize("B,H,N,D,causal", RAGGED)
+def test_ragged_sequence_lengths(lib, B, H, N, D, causal):
+    """No right-padding: any N is accepted and matches the oracle on the same N."""
+    scale = 1.0 / math.sqrt(D)
+    q, k, v, do = ao.make_inputs(B, N, H, D, seed=3 * N + D)
+    print(f"ragged B{B} H{H} N{N} D{D} causal={causal}", flush=True)
+    qg, kg, vg, dog = (t.cuda() for t in (q, k, v, do))
+    out, lse = abi.forward(lib, qg, kg, vg, scale, causal)
+    dq, dk, dv, delta = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal)
+    dq2, dk2, dv2, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal, split=True)
+    torch.cuda.synchronize()
+    o_ref, lse_ref = ao.attention_forward(q, k, v, scale, causal)
+    dq_ref, dk_ref, dv_ref = ao.attention_backward(q, k, v, do, scale, causal)
+    assert _err(out, o_ref) <= O_TOL
+    assert (lse.cpu() - lse_ref).abs().max().item() <= LSE_TOL
+    assert (delta.cpu() - ao.attention_delta(out.cpu(), do)).abs().max().item() <= 1e-3
+    assert _err(dq, dq_ref) <= G_TOL and _err(dk, dk_ref) <= G_TOL and _err(dv, dv_ref) <= G_TOL
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    # the same rows inside a longer, right-padded sequence give the same output under
+    # causal masking (the reference's way of handling such lengths, README.md:3)
+    if causal:
+        pad = (-N) % 32
+        if pad:
+            qp, kp, vp = (torch.cat([t, torch.zeros(B, pad, H, D, dtype=t.dtype)], 1).cuda() for t in (q, k, v))
+            out_p, _ = abi.forward(lib, qp, kp, vp, scale, True)
+            # (not bit for bit: when the running maximum is moved depends on all 32 rows of a wave)
+            assert (out_p[:, :N].float() - out.float()).abs().max().item() <= 1e-3
+
+
 def test_golden_fixtures_on_gpu(lib):
     import os
     import numpy as np
@@ -178,8 +213,8 @@ def test_non_dense_inputs_and_side_stream():
 def test_errors_on_gpu():
     from flash_attn_v100 import flash_attn_func
 
-    bad = torch.zeros(1, 48, 2, 64, dtype=torch.float16, device="cuda")
-    with pytest.raises(RuntimeError, match="multiple of 32"):
+    bad = torch.zeros(1, 0, 2, 64, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="seqlen must be positive"):
         flash_attn_func(bad, bad, bad)
     bad = torch.zeros(1, 64, 2, 32, dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError, match="head dimension"):
