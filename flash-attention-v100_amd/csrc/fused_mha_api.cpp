@@ -10,8 +10,9 @@
 //     in fp32 inside the launcher;
 //   * head size 64 is accepted as well as 128; any seqlen > 0 is accepted (the
 //     reference assumes a multiple of 32, README.md:3, without checking);
-//   * inputs that are not dense (B, N, H, D) are copied dense instead of being
-//     read with wrong strides;
+//   * inputs that are not dense (B, N, H, D) are read through their strides
+//     (or copied dense when the strides do not qualify) instead of being read
+//     with wrong strides;
 //   * the arch gate asks for gfx950 instead of sm_70 (:21-23).
 #include <torch/extension.h>
 #include <c10/core/DeviceGuard.h>
@@ -41,6 +42,25 @@ void check_rc(int rc, const char* what) {
 }
 
 at::Tensor dense(const at::Tensor& x) { return x.is_contiguous() ? x : x.contiguous(); }
+
+// A (batch, seqlen, heads, head_size) input as the kernels take it: the tensor
+// itself with its strides when they qualify (last dimension contiguous, rows on
+// 16-byte boundaries; e.g. a slice of a packed QKV projection or a
+// (batch, heads, seqlen, head_size)-backed view), otherwise a dense copy.  The
+// reference copies (flash_attn_interface.py:14-15) or mis-reads such inputs.
+struct Operand {
+  at::Tensor t;
+  fused_mha_strides st;
+};
+Operand operand(const at::Tensor& x) {
+  const int64_t sb = x.stride(0), sn = x.stride(1), sh = x.stride(2);
+  const bool ok = x.stride(3) == 1 && sb >= 0 && sn >= 0 && sh >= 0 && ((sb | sn | sh) & 7) == 0 &&
+                  sn < (int64_t(1) << 24) && sh < (int64_t(1) << 31) &&
+                  (reinterpret_cast<uintptr_t>(x.data_ptr()) & 15u) == 0;
+  if (ok) return {x, {sb, sn, sh}};
+  at::Tensor c = x.contiguous();
+  return {c, {c.stride(0), c.stride(1), c.stride(2)}};
+}
 
 }  // namespace
 
@@ -86,11 +106,12 @@ std::vector<at::Tensor> mha_fwd(at::Tensor& q,        // batch x seqlen x heads 
   }
 
   c10::DeviceGuard device_guard(q.device());
-  at::Tensor qd = dense(q), kd = dense(k), vd = dense(v);
+  const Operand qo = operand(q), ko = operand(k), vo = operand(v);
   auto lse = torch::empty({batch_size, num_heads, seqlen_q}, q.options().dtype(at::kFloat));
   hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
-  check_rc(fused_mha_forward(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), lse.data_ptr(), batch_size,
-                             num_heads, seqlen_q, seqlen_q, head_size, softmax_scale, is_causal ? 1 : 0, stream),
+  check_rc(fused_mha_forward_strided(qo.t.data_ptr(), &qo.st, ko.t.data_ptr(), &ko.st, vo.t.data_ptr(), &vo.st,
+                                     out.data_ptr(), lse.data_ptr(), batch_size, num_heads, seqlen_q, head_size,
+                                     softmax_scale, is_causal ? 1 : 0, stream),
            "fused_mha_forward");
   return {out, lse};
 }
@@ -147,14 +168,15 @@ std::vector<at::Tensor> mha_bwd(const at::Tensor& dout,  // batch x seqlen x hea
   };
   at::Tensor dq = grad_like(dq_, "dq"), dk = grad_like(dk_, "dk"), dv = grad_like(dv_, "dv");
 
-  at::Tensor qd = dense(q), kd = dense(k), vd = dense(v), od = dense(out), gd = dense(dout), ld = dense(lse);
+  const Operand qo = operand(q), ko = operand(k), vo = operand(v), go = operand(dout);
+  at::Tensor od = dense(out), ld = dense(lse);
   const size_t ws_bytes = fused_mha_backward_workspace_bytes(batch_size, num_heads, seqlen_q, head_size);
   auto workspace = torch::empty({(int64_t)ws_bytes}, q.options().dtype(at::kByte));
   hipStream_t stream = c10::hip::getCurrentHIPStream().stream();
-  check_rc(fused_mha_backward(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), od.data_ptr(), gd.data_ptr(),
-                              ld.data_ptr(), workspace.data_ptr(), ws_bytes, dq.data_ptr(), dk.data_ptr(),
-                              dv.data_ptr(), batch_size, num_heads, seqlen_q, seqlen_q, head_size, softmax_scale,
-                              is_causal ? 1 : 0, stream),
+  check_rc(fused_mha_backward_strided(qo.t.data_ptr(), &qo.st, ko.t.data_ptr(), &ko.st, vo.t.data_ptr(), &vo.st,
+                                      od.data_ptr(), go.t.data_ptr(), &go.st, ld.data_ptr(), workspace.data_ptr(),
+                                      ws_bytes, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), batch_size, num_heads,
+                                      seqlen_q, head_size, softmax_scale, is_causal ? 1 : 0, stream),
            "fused_mha_backward");
   return {dq, dk, dv};
 }

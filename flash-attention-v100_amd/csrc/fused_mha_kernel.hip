@@ -226,6 +226,14 @@ __device__ __forceinline__ void block_barrier() {
 template <int V>
 struct IntTag { static constexpr int value = V; };
 
+// Element strides of a (batch, n, head, d) tensor whose last dimension is
+// contiguous.  The dense layout of reference kernel/fused_mha_kernel.cu:57-59 is
+// {n*head*d, head*d, d}.
+struct Strides {
+  long b;
+  int n, h;
+};
+
 // ---------------------------------------------------------------------------
 // Forward.  Block = 8 waves = 256 queries, wave = 32 queries; K/V tiles of 64
 // keys stream through a 3-slot LDS ring, copied asynchronously two tiles ahead.
@@ -251,7 +259,8 @@ constexpr int kRing = 3;
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(kFwdThreads, 1)
 fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-                half_t* __restrict__ O, float* __restrict__ LSE, int H, int N, int nmb, float c, int negate_q) {
+                Strides qs, Strides ks, Strides vs, half_t* __restrict__ O, float* __restrict__ LSE, int H, int N,
+                int nmb, float c, int negate_q) {
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kFwdWaves;  // copy instructions per wave per tile
@@ -268,11 +277,11 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   slice_and_block(nmb, bh, mb);
   const int mblk = CAUSAL ? nmb - 1 - mb : mb;  // heavy blocks first
   const int b = bh / H, h = bh - b * H;
-  const int rs = H * D;
+  const int rs = H * D;  // O is dense
   const long head_off = ((long)b * N * H + h) * D;
-  const half_t* Qb = Q + head_off;
-  const half_t* Kb = K + head_off;
-  const half_t* Vb = V + head_off;
+  const half_t* Qb = Q + b * qs.b + (long)h * qs.h;
+  const half_t* Kb = K + b * ks.b + (long)h * ks.h;
+  const half_t* Vb = V + b * vs.b + (long)h * vs.h;
 
   const int m0 = mblk * kFwdBlockQ;
   const int q0w = m0 + wave * kResident;
@@ -288,35 +297,37 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   }
 
   // this wave's share of every tile copy
-  int c_row[kIPW], c_goff[kIPW], c_blk[kIPW];
+  int c_row[kIPW], c_kgoff[kIPW], c_vgoff[kIPW], c_blk[kIPW];
 #pragma unroll
   for (int u = 0; u < kIPW; ++u) {
     const int t = wave * kIPW + u;
-    copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
+    copy_src<D>(t, lane, ks.n, c_row[u], c_kgoff[u]);
+    copy_src<D>(t, lane, vs.n, c_row[u], c_vgoff[u]);
     c_blk[u] = t * 1024;
   }
-  auto copy_tile = [&](const half_t* src, char* dst, int tile_idx) __attribute__((always_inline)) {
+  auto copy_tile = [&](const half_t* src, int src_rs, const int (&goff)[kIPW], char* dst, int tile_idx)
+                       __attribute__((always_inline)) {
     const int row0 = tile_idx * kTile;
-    const half_t* tp = src + (long)row0 * rs;  // wave-uniform
+    const half_t* tp = src + (long)row0 * src_rs;  // wave-uniform
     if (row0 + kTile <= N) {
 #pragma unroll
-      for (int u = 0; u < kIPW; ++u) copy16(tp, c_goff[u], dst + c_blk[u]);
+      for (int u = 0; u < kIPW; ++u) copy16(tp, goff[u], dst + c_blk[u]);
     } else {
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) {  // rows past the end re-read row N-1
         const int back = max(row0 + c_row[u] - (N - 1), 0);
-        copy16(tp, c_goff[u] - back * rs * 2, dst + c_blk[u]);
+        copy16(tp, goff[u] - back * src_rs * 2, dst + c_blk[u]);
       }
     }
   };
 
-  copy_tile(Kb, k_ring, 0);
-  if (nt > 1) copy_tile(Kb, k_ring + T::kBytes, 1);
-  copy_tile(Vb, v_ring, 0);
+  copy_tile(Kb, ks.n, c_kgoff, k_ring, 0);
+  if (nt > 1) copy_tile(Kb, ks.n, c_kgoff, k_ring + T::kBytes, 1);
+  copy_tile(Vb, vs.n, c_vgoff, v_ring, 0);
 
   h8 qf[G::kKSteps];
   {
-    const half_t* qp = Qb + (long)min(qi, N - 1) * rs + hh * 8;
+    const half_t* qp = Qb + (long)min(qi, N - 1) * qs.n + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < G::kKSteps; ++kk) {
       qf[kk] = *reinterpret_cast<const h8*>(qp + kk * 16);
@@ -439,8 +450,8 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
       else if (j < nt) wait_vm<kIPW>();
       else wait_vm<0>();
       block_barrier();
-      if (j + 2 < nt) copy_tile(Kb, k_ring + s2 * T::kBytes, j + 2);
-      if (j + 1 < nt) copy_tile(Vb, v_ring + s1 * T::kBytes, j + 1);
+      if (j + 2 < nt) copy_tile(Kb, ks.n, c_kgoff, k_ring + s2 * T::kBytes, j + 2);
+      if (j + 1 < nt) copy_tile(Vb, vs.n, c_vgoff, v_ring + s1 * T::kBytes, j + 1);
       const char* Kl = k_ring + s0 * T::kBytes;
       const char* Vl = v_ring + s2 * T::kBytes;
       if (kFirst) {
@@ -474,26 +485,27 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 // ---------------------------------------------------------------------------
 template <int D>
 __global__ void __launch_bounds__(256)
-fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ dO, const float* __restrict__ LSE,
-                      float* __restrict__ delta, float* __restrict__ lse2, int H, int N, long rows) {
+fmha_bwd_delta_kernel(const half_t* __restrict__ O, const half_t* __restrict__ dO, Strides gs,
+                      const float* __restrict__ LSE, float* __restrict__ delta, float* __restrict__ lse2, int H, int N,
+                      long rows) {
   constexpr int kLanesPerRow = D / 8;
   const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  const long row = t / kLanesPerRow;  // (b*N + n)*H + h
+  const long row = t / kLanesPerRow;  // (b*N + n)*H + h: O is dense, dO has its own strides
   const int c = (int)(t % kLanesPerRow);
+  const long bn = row / H;
+  const int h = (int)(row % H);
+  const long b = bn / N;
+  const int n = (int)(bn % N);
   float acc = 0.f;
   if (row < rows) {
     h8 a = *reinterpret_cast<const h8*>(O + row * D + c * 8);
-    h8 g = *reinterpret_cast<const h8*>(dO + row * D + c * 8);
+    h8 g = *reinterpret_cast<const h8*>(dO + b * gs.b + (long)n * gs.n + (long)h * gs.h + c * 8);
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc = fmaf((float)a[j], (float)g[j], acc);
   }
 #pragma unroll
   for (int off = kLanesPerRow / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
   if (row < rows && c == 0) {
-    const long bn = row / H;
-    const int h = (int)(row % H);
-    const long b = bn / N;
-    const int n = (int)(bn % N);
     const long at = (b * H + h) * N + n;
     delta[at] = acc;
     lse2[at] = LSE[at] * kLog2e;
@@ -528,9 +540,9 @@ constexpr int kDqBlockQ = kDqPairs * kResident;
 template <int D, bool CAUSAL, bool STATS>
 __global__ void __launch_bounds__(kDqThreads, 1)
 fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-                   const half_t* __restrict__ O, const half_t* __restrict__ dO, const float* __restrict__ LSE,
-                   float* __restrict__ delta, float* __restrict__ lse2, half_t* __restrict__ dQ, int H, int N, int nmb,
-                   float c, float scale) {
+                   const half_t* __restrict__ O, const half_t* __restrict__ dO, Strides qs, Strides ks, Strides vs,
+                   Strides gs, const float* __restrict__ LSE, float* __restrict__ delta, float* __restrict__ lse2,
+                   half_t* __restrict__ dQ, int H, int N, int nmb, float c, float scale) {
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kDqWaves;  // copies per wave per tile, per tensor
@@ -550,10 +562,10 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   slice_and_block(nmb, bh, mb);
   const int mblk = CAUSAL ? nmb - 1 - mb : mb;  // heavy blocks first
   const int b = bh / H, h = bh - b * H;
-  const int rs = H * D;
+  const int rs = H * D;  // O and dQ are dense
   const long head_off = ((long)b * N * H + h) * D;
-  const half_t* Kb = K + head_off;
-  const half_t* Vb = V + head_off;
+  const half_t* Kb = K + b * ks.b + (long)h * ks.h;
+  const half_t* Vb = V + b * vs.b + (long)h * vs.h;
 
   const int m0 = mblk * kDqBlockQ;
   const int q0w = m0 + pair * kResident;
@@ -568,34 +580,35 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
     if (q0w >= N) ntw = 0;
   }
 
-  int c_row[kIPW], c_goff[kIPW], c_blk[kIPW];
+  int c_row[kIPW], c_kgoff[kIPW], c_vgoff[kIPW], c_blk[kIPW];
 #pragma unroll
   for (int u = 0; u < kIPW; ++u) {
     const int t = wave * kIPW + u;
-    copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
+    copy_src<D>(t, lane, ks.n, c_row[u], c_kgoff[u]);
+    copy_src<D>(t, lane, vs.n, c_row[u], c_vgoff[u]);
     c_blk[u] = t * 1024;
   }
   auto copy_tiles = [&](int j) __attribute__((always_inline)) {
     const int row0 = j * kTile;
-    const half_t* kp = Kb + (long)row0 * rs;  // wave-uniform
-    const half_t* vp = Vb + (long)row0 * rs;
+    const half_t* kp = Kb + (long)row0 * ks.n;  // wave-uniform
+    const half_t* vp = Vb + (long)row0 * vs.n;
     char* kdst = k_ring + (j & 3) * T::kBytes;
     char* vdst = v_ring + (j % 3) * T::kBytes;
     if (row0 + kTile <= N) {
 #pragma unroll
-      for (int u = 0; u < kIPW; ++u) copy16(kp, c_goff[u], kdst + c_blk[u]);
+      for (int u = 0; u < kIPW; ++u) copy16(kp, c_kgoff[u], kdst + c_blk[u]);
 #pragma unroll
-      for (int u = 0; u < kIPW; ++u) copy16(vp, c_goff[u], vdst + c_blk[u]);
+      for (int u = 0; u < kIPW; ++u) copy16(vp, c_vgoff[u], vdst + c_blk[u]);
     } else {
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) {  // rows past the end re-read row N-1
         const int back = max(row0 + c_row[u] - (N - 1), 0);
-        copy16(kp, c_goff[u] - back * rs * 2, kdst + c_blk[u]);
+        copy16(kp, c_kgoff[u] - back * ks.n * 2, kdst + c_blk[u]);
       }
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) {
         const int back = max(row0 + c_row[u] - (N - 1), 0);
-        copy16(vp, c_goff[u] - back * rs * 2, vdst + c_blk[u]);
+        copy16(vp, c_vgoff[u] - back * vs.n * 2, vdst + c_blk[u]);
       }
     }
   };
@@ -608,7 +621,8 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   const long stat_at = ((long)b * H + h) * N + qrow;
   float stat;
   {
-    const half_t* rp = (role_b ? dO : Q) + head_off + (long)qrow * rs + hh * 8;
+    const half_t* rp = (role_b ? dO + b * gs.b + (long)h * gs.h + (long)qrow * gs.n
+                               : Q + b * qs.b + (long)h * qs.h + (long)qrow * qs.n) + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < G::kKSteps; ++kk) rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
     if (STATS) {
@@ -787,7 +801,8 @@ constexpr int kKvBlockKeys = kKvPairs * kResident;
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(kKvThreads, 1)
 fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-                     const half_t* __restrict__ dO, const float* __restrict__ delta, const float* __restrict__ lse2,
+                     const half_t* __restrict__ dO, Strides qs, Strides ks, Strides vs, Strides gs,
+                     const float* __restrict__ delta, const float* __restrict__ lse2,
                      half_t* __restrict__ dK, half_t* __restrict__ dV, int H, int N, int nnb, float c, float scale) {
   using G = TileGeom<D>;
   using T = SwzTile<D>;
@@ -810,10 +825,10 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   int bh, nblk;
   slice_and_block(nnb, bh, nblk);  // causal: low key blocks are the heavy ones and come first
   const int b = bh / H, h = bh - b * H;
-  const int rs = H * D;
+  const int rs = H * D;  // dK and dV are dense
   const long head_off = ((long)b * N * H + h) * D;
-  const half_t* Qb = Q + head_off;
-  const half_t* dOb = dO + head_off;
+  const half_t* Qb = Q + b * qs.b + (long)h * qs.h;
+  const half_t* dOb = dO + b * gs.b + (long)h * gs.h;
   const float* delta_b = delta + ((long)b * H + h) * N;
   const int lse2_off = (int)(lse2 - delta) * 4;  // bytes from the delta row to the lse2 row; lse2 lies behind delta
 
@@ -827,34 +842,35 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   const int n_it = nt - t_begin;  // >= 1
 
   // this wave's share of every tile copy
-  int c_row[kIPW], c_goff[kIPW], c_blk[kIPW];
+  int c_row[kIPW], c_qgoff[kIPW], c_ggoff[kIPW], c_blk[kIPW];
 #pragma unroll
   for (int u = 0; u < kIPW; ++u) {
     const int t = wave * kIPW + u;
-    copy_src<D>(t, lane, rs, c_row[u], c_goff[u]);
+    copy_src<D>(t, lane, qs.n, c_row[u], c_qgoff[u]);
+    copy_src<D>(t, lane, gs.n, c_row[u], c_ggoff[u]);
     c_blk[u] = t * 1024;
   }
   auto copy_tiles = [&](int it) __attribute__((always_inline)) {  // tile t_begin + it
     const int row0 = (t_begin + it) * kTile;
-    const half_t* qp = Qb + (long)row0 * rs;   // wave-uniform
-    const half_t* gp = dOb + (long)row0 * rs;
+    const half_t* qp = Qb + (long)row0 * qs.n;   // wave-uniform
+    const half_t* gp = dOb + (long)row0 * gs.n;
     char* qdst = q_ring + (it & 3) * T::kBytes;
     char* gdst = g_ring + (it % 3) * T::kBytes;
     if (row0 + kTile <= N) {
 #pragma unroll
-      for (int u = 0; u < kIPW; ++u) copy16(qp, c_goff[u], qdst + c_blk[u]);
+      for (int u = 0; u < kIPW; ++u) copy16(qp, c_qgoff[u], qdst + c_blk[u]);
 #pragma unroll
-      for (int u = 0; u < kIPW; ++u) copy16(gp, c_goff[u], gdst + c_blk[u]);
+      for (int u = 0; u < kIPW; ++u) copy16(gp, c_ggoff[u], gdst + c_blk[u]);
     } else {
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) {  // rows past the end re-read row N-1
         const int back = max(row0 + c_row[u] - (N - 1), 0);
-        copy16(qp, c_goff[u] - back * rs * 2, qdst + c_blk[u]);
+        copy16(qp, c_qgoff[u] - back * qs.n * 2, qdst + c_blk[u]);
       }
 #pragma unroll
       for (int u = 0; u < kIPW; ++u) {
         const int back = max(row0 + c_row[u] - (N - 1), 0);
-        copy16(gp, c_goff[u] - back * rs * 2, gdst + c_blk[u]);
+        copy16(gp, c_ggoff[u] - back * gs.n * 2, gdst + c_blk[u]);
       }
     }
     if (wave == 0) {  // lane l: lse2 and delta of row row0 + l (rows past the end re-read row N-1)
@@ -870,7 +886,8 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   // resident rows of this wave: K for role A, V for role B
   h8 rf[G::kKSteps];
   {
-    const half_t* rp = (role_b ? V : K) + head_off + (long)krow * rs + hh * 8;
+    const half_t* rp = (role_b ? V + b * vs.b + (long)h * vs.h + (long)krow * vs.n
+                               : K + b * ks.b + (long)h * ks.h + (long)krow * ks.n) + hh * 8;
 #pragma unroll
     for (int kk = 0; kk < G::kKSteps; ++kk) {
       rf[kk] = *reinterpret_cast<const h8*>(rp + kk * 16);
@@ -1047,32 +1064,66 @@ int check_shape(int batch, int head, int m, int n, int d) {
 
 bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
 
+// Strides from the C structure, or the dense layout when the caller gave none.
+Strides to_strides(const fused_mha_strides* st, int head, int n, int d) {
+  if (!st) return Strides{(long)n * head * d, head * d, d};
+  return Strides{(long)st->batch, (int)st->seq, (int)st->head};
+}
+
+// Every row must start on a 16-byte boundary (strides in multiples of 8 halves);
+// the per-lane byte offsets inside a 64-row tile are 32-bit.
+bool bad_strides(const fused_mha_strides* st) {
+  if (!st) return false;
+  if (st->batch < 0 || st->seq < 0 || st->head < 0) return true;
+  if ((st->batch | st->seq | st->head) & 7) return true;
+  return st->seq >= (1 << 24) || st->head >= (1LL << 31);
+}
+
 template <int D, bool CAUSAL>
-int launch_forward(const void* q, const void* k, const void* v, void* o, void* lse, int batch, int head, int n,
-                   float scale, hipStream_t stream) {
+int launch_forward(const void* q, const void* k, const void* v, Strides qs, Strides ks, Strides vs, void* o, void* lse,
+                   int batch, int head, int n, float scale, hipStream_t stream) {
   const int nmb = (n + kFwdBlockQ - 1) / kFwdBlockQ;
   dim3 grid(nmb * batch * head);
   // scale == 0 would turn the masked scores (-inf) into NaN when multiplied; a
   // tiny positive factor gives the same uniform softmax and keeps -inf * c = -inf.
   const float c = fmaxf(fabsf(scale) * kLog2e, 1e-30f);
   fmha_fwd_kernel<D, CAUSAL><<<grid, kFwdThreads, 0, stream>>>(
-      (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, (float*)lse, head, n, nmb, c, scale < 0.f ? 1 : 0);
+      (const half_t*)q, (const half_t*)k, (const half_t*)v, qs, ks, vs, (half_t*)o, (float*)lse, head, n, nmb, c,
+      scale < 0.f ? 1 : 0);
   return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
+}
+
+int dispatch_forward(const void* q, const fused_mha_strides* q_st, const void* k, const fused_mha_strides* k_st,
+                     const void* v, const fused_mha_strides* v_st, void* o, void* lse, int batch, int head, int m,
+                     int n, int d, float scale, int causal, void* stream) {
+  if (!q || !k || !v || !o || !lse) return FUSED_MHA_ERR_NULL_POINTER;
+  if (int rc = check_shape(batch, head, m, n, d)) return rc;
+  if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
+  if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(o) || misaligned(lse))
+    return FUSED_MHA_ERR_MISALIGNED;
+  if (bad_strides(q_st) || bad_strides(k_st) || bad_strides(v_st)) return FUSED_MHA_ERR_BAD_STRIDE;
+  hipStream_t s = (hipStream_t)stream;
+  const Strides qs = to_strides(q_st, head, n, d), ks = to_strides(k_st, head, n, d), vs = to_strides(v_st, head, n, d);
+#define FMHA_FWD(DD, CC) launch_forward<DD, CC>(q, k, v, qs, ks, vs, o, lse, batch, head, n, scale, s)
+  if (d == 128) return causal ? FMHA_FWD(128, true) : FMHA_FWD(128, false);
+  return causal ? FMHA_FWD(64, true) : FMHA_FWD(64, false);
+#undef FMHA_FWD
 }
 
 enum BwdPass { kPassDelta = 1, kPassDq = 2, kPassDkDv = 4, kPassAll = 7 };
 
 template <int D, bool CAUSAL>
 int launch_backward(int passes, const void* q, const void* k, const void* v, const void* o, const void* d_o,
-                    const void* lse, float* delta, void* dq, void* dk, void* dv, int batch, int head, int n,
-                    float scale, hipStream_t stream) {
+                    Strides qs, Strides ks, Strides vs, Strides gs, const void* lse, float* delta, void* dq, void* dk,
+                    void* dv, int batch, int head, int n, float scale, hipStream_t stream) {
   // With all three passes asked for, the dQ pass produces delta and lse2 itself.
   const bool dq_makes_stats = (passes & kPassAll) == kPassAll;
   if ((passes & kPassDelta) && !dq_makes_stats) {
     const long rows = (long)batch * n * head;
     const long threads = rows * (D / 8);
     fmha_bwd_delta_kernel<D><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(
-        (const half_t*)o, (const half_t*)d_o, (const float*)lse, delta, delta + (long)batch * head * n, head, n, rows);
+        (const half_t*)o, (const half_t*)d_o, gs, (const float*)lse, delta, delta + (long)batch * head * n, head, n,
+        rows);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   const float c = scale * kLog2e;
@@ -1080,27 +1131,29 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
     const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;
     if (dq_makes_stats)
       fmha_bwd_dq_kernel<D, CAUSAL, true><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
-          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o,
+          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o, qs, ks, vs, gs,
           (const float*)lse, delta, delta + (long)batch * head * n, (half_t*)dq, head, n, nmb, c, scale);
     else
       fmha_bwd_dq_kernel<D, CAUSAL, false><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
-          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o,
+          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o, qs, ks, vs, gs,
           (const float*)lse, delta, delta + (long)batch * head * n, (half_t*)dq, head, n, nmb, c, scale);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   if (passes & kPassDkDv) {
     const int nnb = (n + kKvBlockKeys - 1) / kKvBlockKeys;
     fmha_bwd_dkdv_kernel<D, CAUSAL><<<dim3(nnb * batch * head), kKvThreads, 0, stream>>>(
-        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, delta, delta + (long)batch * head * n,
-        (half_t*)dk, (half_t*)dv, head, n, nnb, c, scale);
+        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, qs, ks, vs, gs, delta,
+        delta + (long)batch * head * n, (half_t*)dk, (half_t*)dv, head, n, nnb, c, scale);
     if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   return FUSED_MHA_OK;
 }
 
-int dispatch_backward(int passes, const void* q, const void* k, const void* v, const void* o, const void* d_o,
-                      const void* lse, void* workspace, size_t workspace_bytes, void* dq, void* dk, void* dv,
-                      int batch, int head, int m, int n, int d, float scale, int causal, void* stream) {
+int dispatch_backward(int passes, const void* q, const fused_mha_strides* q_st, const void* k,
+                      const fused_mha_strides* k_st, const void* v, const fused_mha_strides* v_st, const void* o,
+                      const void* d_o, const fused_mha_strides* g_st, const void* lse, void* workspace,
+                      size_t workspace_bytes, void* dq, void* dk, void* dv, int batch, int head, int m, int n, int d,
+                      float scale, int causal, void* stream) {
   const bool need_o = passes & kPassDelta, need_dq = passes & kPassDq, need_dkdv = passes & kPassDkDv;
   if (!d_o || !workspace || !lse || (need_o && !o) || ((need_dq || need_dkdv) && (!q || !k || !v)) ||
       (need_dq && !dq) || (need_dkdv && (!dk || !dv)))
@@ -1111,10 +1164,13 @@ int dispatch_backward(int passes, const void* q, const void* k, const void* v, c
   if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(o) || misaligned(d_o) || misaligned(lse) ||
       misaligned(workspace) || misaligned(dq) || misaligned(dk) || misaligned(dv))
     return FUSED_MHA_ERR_MISALIGNED;
+  if (bad_strides(q_st) || bad_strides(k_st) || bad_strides(v_st) || bad_strides(g_st)) return FUSED_MHA_ERR_BAD_STRIDE;
   hipStream_t s = (hipStream_t)stream;
   float* delta = (float*)workspace;
+  const Strides qs = to_strides(q_st, head, n, d), ks = to_strides(k_st, head, n, d),
+                vs = to_strides(v_st, head, n, d), gs = to_strides(g_st, head, n, d);
 #define FMHA_BWD(DD, CC) \
-  launch_backward<DD, CC>(passes, q, k, v, o, d_o, lse, delta, dq, dk, dv, batch, head, n, scale, s)
+  launch_backward<DD, CC>(passes, q, k, v, o, d_o, qs, ks, vs, gs, lse, delta, dq, dk, dv, batch, head, n, scale, s)
   if (d == 128) return causal ? FMHA_BWD(128, true) : FMHA_BWD(128, false);
   return causal ? FMHA_BWD(64, true) : FMHA_BWD(64, false);
 #undef FMHA_BWD
@@ -1127,19 +1183,16 @@ extern "C" {
 int fused_mha_forward(const void* query_ptr, const void* key_ptr, const void* value_ptr, void* output_ptr,
                       void* lse_ptr, int batch, int head, int m, int n, int d, float scale, int causal,
                       void* stream) {
-  if (!query_ptr || !key_ptr || !value_ptr || !output_ptr || !lse_ptr) return FUSED_MHA_ERR_NULL_POINTER;
-  if (int rc = check_shape(batch, head, m, n, d)) return rc;
-  if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
-  if (misaligned(query_ptr) || misaligned(key_ptr) || misaligned(value_ptr) || misaligned(output_ptr) ||
-      misaligned(lse_ptr))
-    return FUSED_MHA_ERR_MISALIGNED;
-  hipStream_t s = (hipStream_t)stream;
-  if (d == 128) {
-    return causal ? launch_forward<128, true>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s)
-                  : launch_forward<128, false>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s);
-  }
-  return causal ? launch_forward<64, true>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s)
-                : launch_forward<64, false>(query_ptr, key_ptr, value_ptr, output_ptr, lse_ptr, batch, head, n, scale, s);
+  return dispatch_forward(query_ptr, nullptr, key_ptr, nullptr, value_ptr, nullptr, output_ptr, lse_ptr, batch, head,
+                          m, n, d, scale, causal, stream);
+}
+
+int fused_mha_forward_strided(const void* query_ptr, const fused_mha_strides* query_strides, const void* key_ptr,
+                              const fused_mha_strides* key_strides, const void* value_ptr,
+                              const fused_mha_strides* value_strides, void* output_ptr, void* lse_ptr, int batch,
+                              int head, int n, int d, float scale, int causal, void* stream) {
+  return dispatch_forward(query_ptr, query_strides, key_ptr, key_strides, value_ptr, value_strides, output_ptr,
+                          lse_ptr, batch, head, n, n, d, scale, causal, stream);
 }
 
 size_t fused_mha_backward_workspace_bytes(int batch, int head, int n, int d) {
@@ -1151,32 +1204,46 @@ int fused_mha_backward(const void* query_ptr, const void* key_ptr, const void* v
                        const void* d_output_ptr, const void* lse_ptr, void* workspace, size_t workspace_bytes,
                        void* d_query_ptr, void* d_key_ptr, void* d_value_ptr, int batch, int head, int m, int n,
                        int d, float scale, int causal, void* stream) {
-  return dispatch_backward(kPassAll, query_ptr, key_ptr, value_ptr, output_ptr, d_output_ptr, lse_ptr, workspace,
-                           workspace_bytes, d_query_ptr, d_key_ptr, d_value_ptr, batch, head, m, n, d, scale, causal,
-                           stream);
+  return dispatch_backward(kPassAll, query_ptr, nullptr, key_ptr, nullptr, value_ptr, nullptr, output_ptr,
+                           d_output_ptr, nullptr, lse_ptr, workspace, workspace_bytes, d_query_ptr, d_key_ptr,
+                           d_value_ptr, batch, head, m, n, d, scale, causal, stream);
+}
+
+int fused_mha_backward_strided(const void* query_ptr, const fused_mha_strides* query_strides, const void* key_ptr,
+                               const fused_mha_strides* key_strides, const void* value_ptr,
+                               const fused_mha_strides* value_strides, const void* output_ptr,
+                               const void* d_output_ptr, const fused_mha_strides* d_output_strides,
+                               const void* lse_ptr, void* workspace, size_t workspace_bytes, void* d_query_ptr,
+                               void* d_key_ptr, void* d_value_ptr, int batch, int head, int n, int d, float scale,
+                               int causal, void* stream) {
+  return dispatch_backward(kPassAll, query_ptr, query_strides, key_ptr, key_strides, value_ptr, value_strides,
+                           output_ptr, d_output_ptr, d_output_strides, lse_ptr, workspace, workspace_bytes,
+                           d_query_ptr, d_key_ptr, d_value_ptr, batch, head, n, n, d, scale, causal, stream);
 }
 
 int fused_mha_backward_delta(const void* output_ptr, const void* d_output_ptr, const void* lse_ptr, void* workspace,
                              size_t workspace_bytes, int batch, int head, int n, int d, void* stream) {
-  return dispatch_backward(kPassDelta, nullptr, nullptr, nullptr, output_ptr, d_output_ptr, lse_ptr, workspace,
-                           workspace_bytes, nullptr, nullptr, nullptr, batch, head, n, n, d, 1.f, 0, stream);
+  return dispatch_backward(kPassDelta, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, output_ptr, d_output_ptr,
+                           nullptr, lse_ptr, workspace, workspace_bytes, nullptr, nullptr, nullptr, batch, head, n, n,
+                           d, 1.f, 0, stream);
 }
 
 int fused_mha_backward_dq(const void* query_ptr, const void* key_ptr, const void* value_ptr,
                           const void* d_output_ptr, const void* lse_ptr, void* workspace, size_t workspace_bytes,
                           void* d_query_ptr, int batch, int head, int n, int d, float scale, int causal,
                           void* stream) {
-  return dispatch_backward(kPassDq, query_ptr, key_ptr, value_ptr, nullptr, d_output_ptr, lse_ptr, workspace,
-                           workspace_bytes, d_query_ptr, nullptr, nullptr, batch, head, n, n, d, scale, causal, stream);
+  return dispatch_backward(kPassDq, query_ptr, nullptr, key_ptr, nullptr, value_ptr, nullptr, nullptr, d_output_ptr,
+                           nullptr, lse_ptr, workspace, workspace_bytes, d_query_ptr, nullptr, nullptr, batch, head, n,
+                           n, d, scale, causal, stream);
 }
 
 int fused_mha_backward_dkdv(const void* query_ptr, const void* key_ptr, const void* value_ptr,
                             const void* d_output_ptr, const void* lse_ptr, void* workspace, size_t workspace_bytes,
                             void* d_key_ptr, void* d_value_ptr, int batch, int head, int n, int d, float scale,
                             int causal, void* stream) {
-  return dispatch_backward(kPassDkDv, query_ptr, key_ptr, value_ptr, nullptr, d_output_ptr, lse_ptr, workspace,
-                           workspace_bytes, nullptr, d_key_ptr, d_value_ptr, batch, head, n, n, d, scale, causal,
-                           stream);
+  return dispatch_backward(kPassDkDv, query_ptr, nullptr, key_ptr, nullptr, value_ptr, nullptr, nullptr, d_output_ptr,
+                           nullptr, lse_ptr, workspace, workspace_bytes, nullptr, d_key_ptr, d_value_ptr, batch, head,
+                           n, n, d, scale, causal, stream);
 }
 
 const char* fused_mha_error_string(int code) {
@@ -1189,6 +1256,8 @@ const char* fused_mha_error_string(int code) {
     case FUSED_MHA_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";
     case FUSED_MHA_ERR_BAD_SCALE: return "scale must be finite";
     case FUSED_MHA_ERR_TOO_LARGE: return "batch * head exceeds 65535";
+    case FUSED_MHA_ERR_BAD_STRIDE:
+      return "strides must be non-negative multiples of 8 elements, sequence stride below 2^24, head stride below 2^31";
     default: return "unknown fused_mha error code";
   }
 }

@@ -42,6 +42,20 @@ extern "C" {
 #define FUSED_MHA_ERR_LAUNCH (-5)         /* the HIP runtime refused the launch    */
 #define FUSED_MHA_ERR_BAD_SCALE (-6)      /* scale is NaN or infinite              */
 #define FUSED_MHA_ERR_TOO_LARGE (-7)      /* batch*head exceeds the grid limit     */
+#define FUSED_MHA_ERR_BAD_STRIDE (-8)     /* see fused_mha_strides                 */
+
+/*
+ * Element strides of a (batch, n, head, d) tensor whose last dimension is
+ * contiguous: element (b, i, h, j) sits at b*batch + i*seq + h*head + j.
+ * The dense layout is {n*head*d, head*d, d}.  Each stride must be a
+ * non-negative multiple of 8 (rows start on 16-byte boundaries), seq below
+ * 2^24 and head below 2^31.
+ */
+typedef struct fused_mha_strides {
+  long long batch;
+  long long seq;
+  long long head;
+} fused_mha_strides;
 
 /*
  * Forward: o = softmax(scale * q k^T  [+ causal mask]) v, lse = row logsumexp.
@@ -53,6 +67,22 @@ int fused_mha_forward(const void *query_ptr, const void *key_ptr, const void *va
                       void *output_ptr, void *lse_ptr,
                       int batch, int head, int m, int n, int d,
                       float scale, int causal, void *stream);
+
+/*
+ * The same for inputs that are not dense: q, k and v each come with their own
+ * strides (NULL = dense), e.g. the three slices of a packed (batch, n, 3, head,
+ * d) projection or (batch, head, n, d)-backed views; o and lse are written
+ * dense.  No counterpart in the reference, whose Python side copies such inputs
+ * (flash_attn_interface.py:14-15) and whose kernel assumes the dense layout
+ * (kernel/fused_mha_kernel.cu:57-59); it is for callers that want to skip that
+ * copy.
+ */
+int fused_mha_forward_strided(const void *query_ptr, const fused_mha_strides *query_strides,
+                              const void *key_ptr, const fused_mha_strides *key_strides,
+                              const void *value_ptr, const fused_mha_strides *value_strides,
+                              void *output_ptr, void *lse_ptr,
+                              int batch, int head, int n, int d,
+                              float scale, int causal, void *stream);
 
 /*
  * Bytes of device scratch fused_mha_backward needs for this problem size
@@ -77,6 +107,21 @@ int fused_mha_backward(const void *query_ptr, const void *key_ptr, const void *v
                        void *d_query_ptr, void *d_key_ptr, void *d_value_ptr,
                        int batch, int head, int m, int n, int d,
                        float scale, int causal, void *stream);
+
+/*
+ * The same with strides for q, k, v and d_o (NULL = dense); o, lse, d_q, d_k
+ * and d_v are dense.  No counterpart in the reference (see
+ * fused_mha_forward_strided).
+ */
+int fused_mha_backward_strided(const void *query_ptr, const fused_mha_strides *query_strides,
+                               const void *key_ptr, const fused_mha_strides *key_strides,
+                               const void *value_ptr, const fused_mha_strides *value_strides,
+                               const void *output_ptr,
+                               const void *d_output_ptr, const fused_mha_strides *d_output_strides,
+                               const void *lse_ptr, void *workspace, size_t workspace_bytes,
+                               void *d_query_ptr, void *d_key_ptr, void *d_value_ptr,
+                               int batch, int head, int n, int d,
+                               float scale, int causal, void *stream);
 
 /*
  * The three passes fused_mha_backward enqueues, one entry point each, so a

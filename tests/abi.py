@@ -14,10 +14,22 @@ LIB_PATH = os.path.join(ROOT, "flash-attention-v100_amd", "lib", "libfused_mha.s
 HEADER = os.path.join(ROOT, "include", "fused_mha.h")
 
 OK = 0
-ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_BAD_HEAD_DIM, ERR_MISALIGNED, ERR_LAUNCH, ERR_BAD_SCALE, ERR_TOO_LARGE = (
-    -1, -2, -3, -4, -5, -6, -7)
+(ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_BAD_HEAD_DIM, ERR_MISALIGNED, ERR_LAUNCH, ERR_BAD_SCALE, ERR_TOO_LARGE,
+ ERR_BAD_STRIDE) = (-1, -2, -3, -4, -5, -6, -7, -8)
 
 _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+
+
+class Strides(ctypes.Structure):
+    """struct fused_mha_strides: element strides of a (batch, n, head, d) tensor."""
+    _fields_ = [("batch", ctypes.c_longlong), ("seq", ctypes.c_longlong), ("head", ctypes.c_longlong)]
+
+    @classmethod
+    def of(cls, t):
+        return cls(t.stride(0), t.stride(1), t.stride(2))
+
+
+_sp = ctypes.POINTER(Strides)
 
 
 def declared_symbols():
@@ -43,6 +55,11 @@ def load():
     lib.fused_mha_backward_dq.restype = _i
     lib.fused_mha_backward_dkdv.argtypes = [_vp] * 6 + [_sz, _vp, _vp] + [_i] * 4 + [_f, _i, _vp]
     lib.fused_mha_backward_dkdv.restype = _i
+    lib.fused_mha_forward_strided.argtypes = [_vp, _sp] * 3 + [_vp, _vp] + [_i] * 4 + [_f, _i, _vp]
+    lib.fused_mha_forward_strided.restype = _i
+    lib.fused_mha_backward_strided.argtypes = ([_vp, _sp] * 3 + [_vp, _vp, _sp, _vp, _vp, _sz] + [_vp] * 3 + [_i] * 4 +
+                                               [_f, _i, _vp])
+    lib.fused_mha_backward_strided.restype = _i
     lib.fused_mha_error_string.argtypes = [_i]
     lib.fused_mha_error_string.restype = ctypes.c_char_p
     return lib
@@ -81,3 +98,30 @@ def backward(lib, q, k, v, out, dout, lse, scale, causal, stream=None, split=Fal
                                     dv.data_ptr(), B, H, N, N, D, scale, int(causal), s)
     assert rc == OK, lib.fused_mha_error_string(rc)
     return dq, dk, dv, ws.view(torch.float32)[:B * H * N].view(B, H, N)
+
+
+def forward_strided(lib, q, k, v, scale, causal):
+    """q, k, v: fp16 device tensors (B, N, H, D) with any qualifying strides.  Returns dense (out, lse)."""
+    B, N, H, D = q.shape
+    out = torch.empty((B, N, H, D), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+    s = torch.cuda.current_stream().cuda_stream
+    rc = lib.fused_mha_forward_strided(q.data_ptr(), Strides.of(q), k.data_ptr(), Strides.of(k), v.data_ptr(),
+                                       Strides.of(v), out.data_ptr(), lse.data_ptr(), B, H, N, D, scale, int(causal), s)
+    assert rc == OK, lib.fused_mha_error_string(rc)
+    return out, lse
+
+
+def backward_strided(lib, q, k, v, out, dout, lse, scale, causal):
+    """q, k, v, dout with any qualifying strides; out, lse dense.  Returns dense (dq, dk, dv)."""
+    B, N, H, D = q.shape
+    nbytes = lib.fused_mha_backward_workspace_bytes(B, H, N, D)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    dq, dk, dv = (torch.empty((B, N, H, D), dtype=q.dtype, device=q.device) for _ in range(3))
+    s = torch.cuda.current_stream().cuda_stream
+    rc = lib.fused_mha_backward_strided(q.data_ptr(), Strides.of(q), k.data_ptr(), Strides.of(k), v.data_ptr(),
+                                        Strides.of(v), out.data_ptr(), dout.data_ptr(), Strides.of(dout),
+                                        lse.data_ptr(), ws.data_ptr(), nbytes, dq.data_ptr(), dk.data_ptr(),
+                                        dv.data_ptr(), B, H, N, D, scale, int(causal), s)
+    assert rc == OK, lib.fused_mha_error_string(rc)
+    return dq, dk, dv

@@ -20,14 +20,14 @@ def test_exports_every_declared_symbol(lib):
     names = abi.declared_symbols()
     assert names == sorted(["fused_mha_forward", "fused_mha_backward", "fused_mha_backward_workspace_bytes",
                             "fused_mha_backward_delta", "fused_mha_backward_dq", "fused_mha_backward_dkdv",
-                            "fused_mha_error_string"])
+                            "fused_mha_forward_strided", "fused_mha_backward_strided", "fused_mha_error_string"])
     for name in names:
         assert hasattr(lib, name), name
 
 
 def test_error_strings(lib):
     seen = set()
-    for code in range(0, -8, -1):
+    for code in range(0, -9, -1):
         text = lib.fused_mha_error_string(code).decode()
         assert text and text not in seen
         seen.add(text)
@@ -70,6 +70,26 @@ def test_backward_validation_codes(lib):
     assert lib.fused_mha_backward_delta(p, None, p, p, ws, 1, 1, 32, 64, None) == abi.ERR_NULL_POINTER
     assert lib.fused_mha_backward_dq(p, p, p, p, p, p, ws, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
     assert lib.fused_mha_backward_dkdv(p, p, p, p, p, p, ws, p, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+
+
+def test_strided_validation_codes(lib):
+    p = 0x1000  # never dereferenced: every call below is rejected before a launch
+    f = lib.fused_mha_forward_strided
+    ok = abi.Strides(32 * 2 * 64, 2 * 64, 64)
+
+    def call(qs, ks=ok, vs=ok):
+        return f(p, qs, p, ks, p, vs, p, p, 1, 2, 32, 64, 1.0, 0, None)
+
+    assert call(abi.Strides(32 * 2 * 64, 2 * 64, 68)) == abi.ERR_BAD_STRIDE      # rows off 16-byte boundaries
+    assert call(ok, abi.Strides(-4096, 128, 64)) == abi.ERR_BAD_STRIDE           # negative
+    assert call(ok, ok, abi.Strides(1 << 30, 1 << 24, 64)) == abi.ERR_BAD_STRIDE  # sequence stride too large
+    assert f(None, ok, p, ok, p, ok, p, p, 1, 2, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+    assert f(p, ok, p, ok, p, ok, p, p, 1, 2, 32, 96, 1.0, 0, None) == abi.ERR_BAD_HEAD_DIM
+    g = lib.fused_mha_backward_strided
+    bad = abi.Strides(4096, 130, 64)
+    assert g(p, ok, p, ok, p, ok, p, p, bad, p, p, 1 << 20, p, p, p, 1, 2, 32, 64, 1.0, 0, None) == abi.ERR_BAD_STRIDE
+    assert g(p, ok, p, ok, p, ok, p, p, ok, p, p, 8, p, p, p, 1, 2, 32, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE  # workspace
+    assert b"stride" in lib.fused_mha_error_string(abi.ERR_BAD_STRIDE)
 
 
 def test_python_api_signature():

@@ -210,6 +210,61 @@ def test_non_dense_inputs_and_side_stream():
     assert _err(qg.grad, dq_ref) <= G_TOL and _err(kg.grad, dk_ref) <= G_TOL and _err(vg.grad, dv_ref) <= G_TOL
 
 
+def _strided_cases(B, N, H, D, seed):
+    """The same values behind three layouts that are not dense (B, N, H, D)."""
+    q, k, v, do = ao.make_inputs(B, N, H, D, seed=seed)
+    packed = torch.stack([q, k, v], dim=2).cuda()                      # (B, N, 3, H, D): a fused QKV projection
+    heads_first = [t.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3) for t in (q, k, v, do)]  # (B, H, N, D) storage
+    wide = [torch.cat([t, t], dim=3).cuda()[..., :D] for t in (q, k, v, do)]   # rows twice as long as D
+    return (q, k, v, do), {
+        "packed_qkv": (packed[:, :, 0], packed[:, :, 1], packed[:, :, 2], do.cuda()),
+        "heads_first": tuple(heads_first),
+        "wide_rows": tuple(wide),
+    }
+
+
+@pytest.mark.parametrize("B,H,N,D,causal", [(2, 3, 200, 64, True), (1, 2, 320, 128, False), (2, 2, 96, 128, True)])
+def test_strided_inputs_c_abi(lib, B, H, N, D, causal):
+    """Strided q, k, v, dout give the same bits as their dense copies, without a copy."""
+    scale = 1.0 / math.sqrt(D)
+    (q, k, v, do), cases = _strided_cases(B, N, H, D, seed=N + D + 1)
+    qd, kd, vd, dod = (t.cuda() for t in (q, k, v, do))
+    out_d, lse_d = abi.forward(lib, qd, kd, vd, scale, causal)
+    dq_d, dk_d, dv_d, _ = abi.backward(lib, qd, kd, vd, out_d, dod, lse_d, scale, causal)
+    o_ref, _ = ao.attention_forward(q, k, v, scale, causal)
+    assert _err(out_d, o_ref) <= O_TOL
+    for name, (qs, ks, vs, gs) in cases.items():
+        print(f"strided {name} B{B} H{H} N{N} D{D} causal={causal} q.stride={tuple(qs.stride())}", flush=True)
+        assert not qs.is_contiguous() and torch.equal(qs, qd)
+        out, lse = abi.forward_strided(lib, qs, ks, vs, scale, causal)
+        dq, dk, dv = abi.backward_strided(lib, qs, ks, vs, out, gs, lse, scale, causal)
+        torch.cuda.synchronize()
+        assert torch.equal(out, out_d) and torch.equal(lse, lse_d), name
+        assert torch.equal(dq, dq_d) and torch.equal(dk, dk_d) and torch.equal(dv, dv_d), name
+
+
+def test_strided_inputs_python_api():
+    """flash_attn_func on views of a packed QKV tensor: gradients flow back into the packed tensor."""
+    from flash_attn_v100 import flash_attn_func
+
+    B, H, N, D = 2, 4, 160, 64
+    q, k, v, do = ao.make_inputs(B, N, H, D, seed=77)
+    packed = torch.stack([q, k, v], dim=2).cuda().requires_grad_()
+    out = flash_attn_func(packed[:, :, 0], packed[:, :, 1], packed[:, :, 2], None, True)
+    out.backward(do.cuda())
+    scale = 1.0 / math.sqrt(D)
+    o_ref, _ = ao.attention_forward(q, k, v, scale, True)
+    dq_ref, dk_ref, dv_ref = ao.attention_backward(q, k, v, do, scale, True)
+    assert _err(out, o_ref) <= O_TOL
+    g = packed.grad
+    assert _err(g[:, :, 0], dq_ref) <= G_TOL and _err(g[:, :, 1], dk_ref) <= G_TOL and _err(g[:, :, 2], dv_ref) <= G_TOL
+    # a layout whose rows are not on 16-byte boundaries falls back to a dense copy and still works
+    odd = torch.zeros(B, N, H, D + 4, dtype=torch.float16, device="cuda")
+    odd[..., :D] = q.cuda()
+    out2 = flash_attn_func(odd[..., :D], k.cuda(), v.cuda(), None, True)
+    assert torch.equal(out2, out.detach())
+
+
 def test_errors_on_gpu():
     from flash_attn_v100 import flash_attn_func
 
