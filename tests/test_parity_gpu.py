@@ -210,6 +210,31 @@ def test_non_dense_inputs_and_side_stream():
     assert _err(qg.grad, dq_ref) <= G_TOL and _err(kg.grad, dk_ref) <= G_TOL and _err(vg.grad, dv_ref) <= G_TOL
 
 
+@pytest.mark.parametrize("D,causal", [(64, True), (128, False), (128, True)])
+def test_wide_score_ranges(lib, D, causal):
+    """Scores whose running maximum keeps growing along the keys and rows dominated by
+    one key: the lazily moved running maximum must still give the oracle's result."""
+    B, H, N = 1, 2, 1024
+    scale = 1.0 / math.sqrt(D)
+    q, k, v, do = ao.make_inputs(B, N, H, D, seed=11 + D)
+    ramp = torch.linspace(0.25, 6.0, N).view(1, N, 1, 1)
+    k = (k.float() * ramp).half()                 # later keys score higher and higher
+    k[:, 0] = (q[:, N // 2].float() * 2).half()   # key 0 is a sink for query N/2
+    q[:, 5] = 0                                   # an all-zero query: uniform attention
+    qg, kg, vg, dog = (t.cuda() for t in (q, k, v, do))
+    out, lse = abi.forward(lib, qg, kg, vg, scale, causal)
+    dq, dk, dv, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal)
+    torch.cuda.synchronize()
+    o_ref, lse_ref = ao.attention_forward(q, k, v, scale, causal)
+    dq_ref, dk_ref, dv_ref = ao.attention_backward(q, k, v, do, scale, causal)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert _err(out, o_ref) <= O_TOL
+    assert (lse.cpu() - lse_ref).abs().max().item() <= LSE_TOL
+    # dQ scales with the keys here (values beyond 16): allow two fp16 steps at its largest magnitude
+    dq_tol = max(G_TOL, 2 * 2.0 ** -10 * dq_ref.abs().max().item())
+    assert _err(dq, dq_ref) <= dq_tol and _err(dk, dk_ref) <= G_TOL and _err(dv, dv_ref) <= G_TOL
+
+
 def _strided_cases(B, N, H, D, seed):
     """The same values behind three layouts that are not dense (B, N, H, D)."""
     q, k, v, do = ao.make_inputs(B, N, H, D, seed=seed)
