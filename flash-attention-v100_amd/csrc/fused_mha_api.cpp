@@ -131,9 +131,12 @@ std::vector<at::Tensor> mha_bwd(const at::Tensor& dout,  // batch x seqlen x hea
   TORCH_CHECK(lse.dtype() == torch::kFloat32, "lse must be fp32");
 
   TORCH_CHECK(q.dim() == 4, "query must have 4 dimensions (batch, seqlen, heads, head_size)");
+  TORCH_CHECK(k.dim() == 4 && v.dim() == 4, "key and value must have 4 dimensions");
+  TORCH_CHECK(out.dim() == 4 && dout.dim() == 4, "out and dout must have 4 dimensions");
   TORCH_CHECK(q.stride(-1) == 1, "Input tensor must have contiguous last dimension");
   TORCH_CHECK(k.stride(-1) == 1, "Input tensor must have contiguous last dimension");
   TORCH_CHECK(v.stride(-1) == 1, "Input tensor must have contiguous last dimension");
+  TORCH_CHECK(dout.stride(-1) == 1, "Input tensor must have contiguous last dimension");
 
   const auto sizes = q.sizes();
   const int batch_size = sizes[0];

@@ -32,8 +32,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <math.h>
+#include <tuple>
 
 #include "fused_mha.h"
+#include "block_map.h"
 
 namespace {
 
@@ -96,24 +98,8 @@ __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long r
   }
 }
 
-// Work-group id -> (batch*head slice, block inside the slice).  Consecutive
-// work-group ids go round-robin over the 8 XCDs, each with a private L2; the
-// remap hands every XCD whole (batch, head) slices, so the blocks that stream
-// the same K/V (or Q/dO) rows share one L2.  Inside an XCD the blocks are
-// ordered block-index major over its slices: callers number blocks heaviest
-// first, so under causal masking all heavy blocks start before any light one
-// (longest-processing-time-first), which keeps the tail of the launch short.
 __device__ __forceinline__ void slice_and_block(int blocks_per_slice, int& slice, int& blk) {
-  const int lin = blockIdx.x, total = gridDim.x;
-  const int slices = total / blocks_per_slice;
-  if ((slices & 7) == 0) {
-    const int xcd = lin & 7, slot = lin >> 3, spx = slices >> 3;  // slices per XCD
-    blk = slot / spx;
-    slice = xcd * spx + (slot - blk * spx);
-  } else {
-    slice = lin / blocks_per_slice;
-    blk = lin - slice * blocks_per_slice;
-  }
+  fmha_slice_and_block(blockIdx.x, gridDim.x / blocks_per_slice, blocks_per_slice, slice, blk);
 }
 
 // ---------------------------------------------------------------------------
@@ -152,13 +138,20 @@ __device__ __forceinline__ void copy_src(int t, int lane, int row_stride, int& r
 // LDS reads wait for it (it cannot tell the ring slots apart and would wait for
 // every copy in flight); the waits for these copies are the explicit wait_vm<>
 // calls in the kernels.  tile_base and lds_block must be wave-uniform.
+// The LDS address travels in m0, which the compiler reserves for itself and
+// does not accept as a clobber: the statement saves and restores it, so a value
+// the compiler keeps there (indirect register indexing, its own LDS copies)
+// survives.
 __device__ __forceinline__ void copy16(const half_t* tile_base, int voff, char* lds_block) {
   const unsigned lds_addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds_block;
+  unsigned saved_m0;
   asm volatile(
-      "s_mov_b32 m0, %2\n\t"
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %3\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dwordx4 %0, %1"
-      :
+      "global_load_lds_dwordx4 %1, %2\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0)
       : "v"(voff), "s"(tile_base), "s"(lds_addr)
       : "memory");
 }
@@ -167,11 +160,14 @@ __device__ __forceinline__ void copy16(const half_t* tile_base, int voff, char* 
 // dword at base + voff and it lands in LDS at lds_dst + 4 * l.
 __device__ __forceinline__ void copy4(const float* base, int voff, char* lds_dst) {
   const unsigned lds_addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds_dst;
+  unsigned saved_m0;
   asm volatile(
-      "s_mov_b32 m0, %2\n\t"
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %3\n\t"
       "s_nop 0\n\t"
-      "global_load_lds_dword %0, %1"
-      :
+      "global_load_lds_dword %1, %2\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0)
       : "v"(voff), "s"(base), "s"(lds_addr)
       : "memory");
 }
@@ -830,7 +826,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   const half_t* Qb = Q + b * qs.b + (long)h * qs.h;
   const half_t* dOb = dO + b * gs.b + (long)h * gs.h;
   const float* delta_b = delta + ((long)b * H + h) * N;
-  const int lse2_off = (int)(lse2 - delta) * 4;  // bytes from the delta row to the lse2 row; lse2 lies behind delta
+  const float* lse2_b = lse2 + ((long)b * H + h) * N;
 
   const int n0 = nblk * kKvBlockKeys;
   const int k0w = n0 + pair * kResident;
@@ -875,7 +871,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     }
     if (wave == 0) {  // lane l: lse2 and delta of row row0 + l (rows past the end re-read row N-1)
       const int at = min(row0 + lane, N - 1) * 4;
-      copy4(delta_b, at + lse2_off, st_ring + (it % 3) * kStBytes);
+      copy4(lse2_b, at, st_ring + (it % 3) * kStBytes);
       copy4(delta_b, at, st_ring + (it % 3) * kStBytes + 256);
     }
   };
@@ -1055,11 +1051,30 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 // ---------------------------------------------------------------------------
 // Host side: validation and launches.
 // ---------------------------------------------------------------------------
+// Limits of the 32-bit arithmetic in the kernels: a (batch, head) row of lse /
+// delta is addressed with 32-bit byte offsets (n < 2^29), and the 1-D grid of
+// the finest pass (128-row blocks) must fit a launch (below 2^31 work groups).
 int check_shape(int batch, int head, int m, int n, int d) {
   if (batch <= 0 || head <= 0 || n <= 0 || m != n) return FUSED_MHA_ERR_BAD_SHAPE;
   if (d != 64 && d != 128) return FUSED_MHA_ERR_BAD_HEAD_DIM;
-  if ((long)batch * head > 65535) return FUSED_MHA_ERR_TOO_LARGE;
+  if (n >= (1 << 29)) return FUSED_MHA_ERR_TOO_LARGE;
+  const long blocks = (long)((n + 127) / 128) * batch * head;
+  if (blocks >= (1L << 31)) return FUSED_MHA_ERR_TOO_LARGE;
   return FUSED_MHA_OK;
+}
+
+// Launch through the C API: the status returned belongs to this launch alone
+// (the <<<>>> form plus hipGetLastError would also report, and clear, an error
+// left behind by earlier, unrelated work on the thread).
+template <typename... Params, typename... Args>
+hipError_t launch(void (*kernel)(Params...), unsigned grid, unsigned block, hipStream_t stream, Args... args) {
+  static_assert(sizeof...(Params) == sizeof...(Args), "argument count");
+  auto pack = [](Params... p) { return std::tuple<Params...>(p...); };
+  std::tuple<Params...> vals = pack(args...);  // converted to the kernel's parameter types
+  void* ptrs[sizeof...(Params)];
+  int idx = 0;
+  std::apply([&](auto&... v) { ((ptrs[idx++] = (void*)&v), ...); }, vals);
+  return hipLaunchKernel((const void*)kernel, dim3(grid), dim3(block), ptrs, 0, stream);
 }
 
 bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
@@ -1083,14 +1098,14 @@ template <int D, bool CAUSAL>
 int launch_forward(const void* q, const void* k, const void* v, Strides qs, Strides ks, Strides vs, void* o, void* lse,
                    int batch, int head, int n, float scale, hipStream_t stream) {
   const int nmb = (n + kFwdBlockQ - 1) / kFwdBlockQ;
-  dim3 grid(nmb * batch * head);
+  const unsigned grid = (unsigned)nmb * batch * head;
   // scale == 0 would turn the masked scores (-inf) into NaN when multiplied; a
   // tiny positive factor gives the same uniform softmax and keeps -inf * c = -inf.
   const float c = fmaxf(fabsf(scale) * kLog2e, 1e-30f);
-  fmha_fwd_kernel<D, CAUSAL><<<grid, kFwdThreads, 0, stream>>>(
-      (const half_t*)q, (const half_t*)k, (const half_t*)v, qs, ks, vs, (half_t*)o, (float*)lse, head, n, nmb, c,
-      scale < 0.f ? 1 : 0);
-  return hipGetLastError() == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
+  const hipError_t rc = launch(fmha_fwd_kernel<D, CAUSAL>, grid, kFwdThreads, stream, (const half_t*)q,
+                               (const half_t*)k, (const half_t*)v, qs, ks, vs, (half_t*)o, (float*)lse, head, n, nmb, c,
+                               scale < 0.f ? 1 : 0);
+  return rc == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
 }
 
 int dispatch_forward(const void* q, const fused_mha_strides* q_st, const void* k, const fused_mha_strides* k_st,
@@ -1118,33 +1133,29 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
                     void* dv, int batch, int head, int n, float scale, hipStream_t stream) {
   // With all three passes asked for, the dQ pass produces delta and lse2 itself.
   const bool dq_makes_stats = (passes & kPassAll) == kPassAll;
+  float* lse2 = delta + (long)batch * head * n;
   if ((passes & kPassDelta) && !dq_makes_stats) {
     const long rows = (long)batch * n * head;
     const long threads = rows * (D / 8);
-    fmha_bwd_delta_kernel<D><<<(unsigned)((threads + 255) / 256), 256, 0, stream>>>(
-        (const half_t*)o, (const half_t*)d_o, gs, (const float*)lse, delta, delta + (long)batch * head * n, head, n,
-        rows);
-    if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+    if (launch(fmha_bwd_delta_kernel<D>, (unsigned)((threads + 255) / 256), 256, stream, (const half_t*)o,
+               (const half_t*)d_o, gs, (const float*)lse, delta, lse2, head, n, rows) != hipSuccess)
+      return FUSED_MHA_ERR_LAUNCH;
   }
   const float c = scale * kLog2e;
   if (passes & kPassDq) {
     const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;
-    if (dq_makes_stats)
-      fmha_bwd_dq_kernel<D, CAUSAL, true><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
-          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o, qs, ks, vs, gs,
-          (const float*)lse, delta, delta + (long)batch * head * n, (half_t*)dq, head, n, nmb, c, scale);
-    else
-      fmha_bwd_dq_kernel<D, CAUSAL, false><<<dim3(nmb * batch * head), kDqThreads, 0, stream>>>(
-          (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)o, (const half_t*)d_o, qs, ks, vs, gs,
-          (const float*)lse, delta, delta + (long)batch * head * n, (half_t*)dq, head, n, nmb, c, scale);
-    if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+    auto kernel = dq_makes_stats ? fmha_bwd_dq_kernel<D, CAUSAL, true> : fmha_bwd_dq_kernel<D, CAUSAL, false>;
+    if (launch(kernel, (unsigned)nmb * batch * head, kDqThreads, stream, (const half_t*)q, (const half_t*)k,
+               (const half_t*)v, (const half_t*)o, (const half_t*)d_o, qs, ks, vs, gs, (const float*)lse, delta, lse2,
+               (half_t*)dq, head, n, nmb, c, scale) != hipSuccess)
+      return FUSED_MHA_ERR_LAUNCH;
   }
   if (passes & kPassDkDv) {
     const int nnb = (n + kKvBlockKeys - 1) / kKvBlockKeys;
-    fmha_bwd_dkdv_kernel<D, CAUSAL><<<dim3(nnb * batch * head), kKvThreads, 0, stream>>>(
-        (const half_t*)q, (const half_t*)k, (const half_t*)v, (const half_t*)d_o, qs, ks, vs, gs, delta,
-        delta + (long)batch * head * n, (half_t*)dk, (half_t*)dv, head, n, nnb, c, scale);
-    if (hipGetLastError() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+    if (launch(fmha_bwd_dkdv_kernel<D, CAUSAL>, (unsigned)nnb * batch * head, kKvThreads, stream, (const half_t*)q,
+               (const half_t*)k, (const half_t*)v, (const half_t*)d_o, qs, ks, vs, gs, (const float*)delta,
+               (const float*)lse2, (half_t*)dk, (half_t*)dv, head, n, nnb, c, scale) != hipSuccess)
+      return FUSED_MHA_ERR_LAUNCH;
   }
   return FUSED_MHA_OK;
 }
@@ -1255,7 +1266,7 @@ const char* fused_mha_error_string(int code) {
     case FUSED_MHA_ERR_MISALIGNED: return "a pointer is not 16-byte aligned";
     case FUSED_MHA_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";
     case FUSED_MHA_ERR_BAD_SCALE: return "scale must be finite";
-    case FUSED_MHA_ERR_TOO_LARGE: return "batch * head exceeds 65535";
+    case FUSED_MHA_ERR_TOO_LARGE: return "problem too large: need n < 2^29 and ceil(n/128) * batch * head < 2^31";
     case FUSED_MHA_ERR_BAD_STRIDE:
       return "strides must be non-negative multiples of 8 elements, sequence stride below 2^24, head stride below 2^31";
     default: return "unknown fused_mha error code";

@@ -23,7 +23,9 @@
  *     All work is enqueued asynchronously; nothing synchronises.
  *   - All pointers are borrowed device pointers and must be 16-byte aligned.
  *   - Return value: FUSED_MHA_OK (0) or a negative FUSED_MHA_ERR_* code.
- *     Nothing is launched when an error is returned.
+ *     Arguments are validated before anything is launched; only
+ *     FUSED_MHA_ERR_LAUNCH can come back after part of the work (an earlier
+ *     pass of the backward) has been enqueued.
  */
 #ifndef FUSED_MHA_H_
 #define FUSED_MHA_H_
@@ -41,7 +43,7 @@ extern "C" {
 #define FUSED_MHA_ERR_MISALIGNED (-4)     /* a pointer is not 16-byte aligned      */
 #define FUSED_MHA_ERR_LAUNCH (-5)         /* the HIP runtime refused the launch    */
 #define FUSED_MHA_ERR_BAD_SCALE (-6)      /* scale is NaN or infinite              */
-#define FUSED_MHA_ERR_TOO_LARGE (-7)      /* batch*head exceeds the grid limit     */
+#define FUSED_MHA_ERR_TOO_LARGE (-7)      /* n >= 2^29 or more than 2^31-1 blocks  */
 #define FUSED_MHA_ERR_BAD_STRIDE (-8)     /* see fused_mha_strides                 */
 
 /*

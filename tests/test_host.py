@@ -54,7 +54,10 @@ def test_forward_validation_codes(lib):
     assert f(p, p, p, p, p, 1, 1, 32, 32, 64, float("nan"), 0, None) == abi.ERR_BAD_SCALE
     assert f(p, p, p, p, p, 1, 1, 32, 32, 64, float("inf"), 0, None) == abi.ERR_BAD_SCALE
     assert f(p + 2, p, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_MISALIGNED
-    assert f(p, p, p, p, p, 4096, 32, 32, 32, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
+    # the limits of the kernels' 32-bit arithmetic: n < 2^29, ceil(n/128)*batch*head < 2^31
+    assert f(p, p, p, p, p, 1, 1, 1 << 29, 1 << 29, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
+    assert f(p, p, p, p, p, 1 << 12, 1 << 12, 1 << 14, 1 << 14, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
+    assert f(p, p, p, p, p, 2048, 2048, 1 << 16, 1 << 16, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
 
 
 def test_backward_validation_codes(lib):
@@ -132,6 +135,12 @@ def test_extension_checks_raise_runtime_error():
         ext.bwd(ok, ok, ok, ok, ok, lse.half(), None, None, None, 0.125, True)
     with pytest.raises(RuntimeError, match="must have shape"):
         ext.bwd(ok, ok, ok, ok, ok, torch.zeros(1, 32, 2), None, None, None, 0.125, True)
+    with pytest.raises(RuntimeError, match="4 dimensions"):
+        ext.bwd(ok, ok, t(32, 2, 64), ok, ok, lse, None, None, None, 0.125, True)
+    with pytest.raises(RuntimeError, match="4 dimensions"):
+        ext.bwd(ok, ok, ok, t(32, 2, 64), ok, lse, None, None, None, 0.125, True)
+    with pytest.raises(RuntimeError, match="4 dimensions"):
+        ext.bwd(t(2, 64), ok, ok, ok, ok, lse, None, None, None, 0.125, True)
 
 
 def test_python_api_rejects_cpu_tensors():
@@ -140,3 +149,52 @@ def test_python_api_rejects_cpu_tensors():
     q = torch.zeros(1, 32, 2, 64, dtype=torch.float16)
     with pytest.raises(RuntimeError, match="must be on the GPU"):
         flash_attn_func(q, q, q, None, True)
+
+
+def test_block_map_is_a_bijection(tmp_path):
+    """csrc/block_map.h, compiled for the host: every (slice, block) pair is produced exactly once for any slice
+    count (multiples of 8 or not), and with a multiple of 8 every slice stays on one XCD (work-group id mod 8)."""
+    import os
+    import subprocess
+
+    src = tmp_path / "check_block_map.cpp"
+    src.write_text(r'''
+#include <cstdio>
+#include <vector>
+#include "block_map.h"
+int main() {
+  for (int slices = 1; slices <= 83; ++slices)
+    for (int bps = 1; bps <= 37; ++bps) {
+      const int total = slices * bps;
+      std::vector<int> seen(total, 0), xcd_of(slices, -1);
+      int shared = 0;
+      for (int lin = 0; lin < total; ++lin) {
+        int s = -1, b = -1;
+        fmha_slice_and_block(lin, slices, bps, s, b);
+        if (s < 0 || s >= slices || b < 0 || b >= bps) { printf("range %d %d %d\n", slices, bps, lin); return 1; }
+        if (seen[s * bps + b]++) { printf("twice %d %d %d\n", slices, bps, lin); return 1; }
+        if (xcd_of[s] < 0) xcd_of[s] = lin & 7;
+        else if (xcd_of[s] != (lin & 7) && s < (slices & ~7)) ++shared;
+      }
+      if (shared) { printf("slice on two XCDs %d %d\n", slices, bps); return 1; }
+    }
+  // heaviest first inside a slice: block indices of one slice appear in ascending order
+  // (the slices beyond a multiple of 8 are cut into per-XCD runs instead)
+  for (int slices : {8, 12, 64, 80}) {
+    const int bps = 16;
+    std::vector<int> last(slices, -1);
+    for (int lin = 0; lin < slices * bps; ++lin) {
+      int s, b;
+      fmha_slice_and_block(lin, slices, bps, s, b);
+      if (s < (slices & ~7) && b <= last[s]) { printf("order %d %d\n", slices, lin); return 1; }
+      last[s] = b;
+    }
+  }
+  puts("ok");
+  return 0;
+}
+''')
+    inc = os.path.join(abi.ROOT, "flash-attention-v100_amd", "csrc")
+    exe = tmp_path / "check_block_map"
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-I", inc, str(src), "-o", str(exe)])
+    assert subprocess.check_output([str(exe)]).decode().strip() == "ok"
