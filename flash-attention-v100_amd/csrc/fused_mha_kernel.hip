@@ -32,10 +32,17 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <math.h>
+#include <mutex>
 #include <tuple>
 
 #include "fused_mha.h"
 #include "block_map.h"
+
+// Backward workspace of fused_mha_backward_noalloc (delta and lse*log2(e), fp32
+// (batch, head, n) each): lives in the code object, one copy per GPU, so that
+// entry point never allocates.  Host code must not use this name as an address;
+// it asks the runtime for the device address once per device (scratch_for_device).
+static __device__ __align__(256) unsigned char scratch[2 * (size_t)FUSED_MHA_NOALLOC_MAX_ROWS * sizeof(float)];
 
 namespace {
 
@@ -1187,6 +1194,24 @@ int dispatch_backward(int passes, const void* q, const fused_mha_strides* q_st, 
 #undef FMHA_BWD
 }
 
+// Device address of `scratch` on the current device, looked up on the first call
+// per device (each GPU holds its own copy of the array at its own address).
+constexpr int kMaxDevices = 64;
+int scratch_for_device(void** out) {
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FUSED_MHA_ERR_RUNTIME;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return FUSED_MHA_ERR_RUNTIME;
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return FUSED_MHA_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1217,6 +1242,23 @@ int fused_mha_backward(const void* query_ptr, const void* key_ptr, const void* v
                        int d, float scale, int causal, void* stream) {
   return dispatch_backward(kPassAll, query_ptr, nullptr, key_ptr, nullptr, value_ptr, nullptr, output_ptr,
                            d_output_ptr, nullptr, lse_ptr, workspace, workspace_bytes, d_query_ptr, d_key_ptr,
+                           d_value_ptr, batch, head, m, n, d, scale, causal, stream);
+}
+
+int fused_mha_backward_noalloc(const void* query_ptr, const void* key_ptr, const void* value_ptr,
+                               const void* output_ptr, const void* d_output_ptr, const void* lse_ptr,
+                               void* d_query_ptr, void* d_key_ptr, void* d_value_ptr, int batch, int head, int m,
+                               int n, int d, float scale, int causal, void* stream) {
+  if (int rc = check_shape(batch, head, m, n, d)) return rc;
+  const size_t rows = (size_t)batch * head * n;
+  if (rows > (size_t)FUSED_MHA_NOALLOC_MAX_ROWS) return FUSED_MHA_ERR_SCRATCH_LIMIT;
+  void* ws = nullptr;
+  if (int rc = scratch_for_device(&ws)) return rc;
+  // Every workspace element the dK/dV pass reads is written by the dQ pass of
+  // the same call (rows 0 .. batch*head*n-1 of both halves), so nothing from
+  // an earlier call is ever read and nothing needs clearing.
+  return dispatch_backward(kPassAll, query_ptr, nullptr, key_ptr, nullptr, value_ptr, nullptr, output_ptr,
+                           d_output_ptr, nullptr, lse_ptr, ws, 2 * rows * sizeof(float), d_query_ptr, d_key_ptr,
                            d_value_ptr, batch, head, m, n, d, scale, causal, stream);
 }
 
@@ -1269,6 +1311,9 @@ const char* fused_mha_error_string(int code) {
     case FUSED_MHA_ERR_TOO_LARGE: return "problem too large: need n < 2^29 and ceil(n/128) * batch * head < 2^31";
     case FUSED_MHA_ERR_BAD_STRIDE:
       return "strides must be non-negative multiples of 8 elements, sequence stride below 2^24, head stride below 2^31";
+    case FUSED_MHA_ERR_SCRATCH_LIMIT:
+      return "batch * head * n exceeds FUSED_MHA_NOALLOC_MAX_ROWS, the size of the static scratch";
+    case FUSED_MHA_ERR_RUNTIME: return "a HIP runtime query failed (current device, scratch address)";
     default: return "unknown fused_mha error code";
   }
 }

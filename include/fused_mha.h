@@ -45,6 +45,11 @@ extern "C" {
 #define FUSED_MHA_ERR_BAD_SCALE (-6)      /* scale is NaN or infinite              */
 #define FUSED_MHA_ERR_TOO_LARGE (-7)      /* n >= 2^29 or more than 2^31-1 blocks  */
 #define FUSED_MHA_ERR_BAD_STRIDE (-8)     /* see fused_mha_strides                 */
+#define FUSED_MHA_ERR_SCRATCH_LIMIT (-9)  /* see fused_mha_backward_noalloc        */
+#define FUSED_MHA_ERR_RUNTIME (-10)       /* a HIP runtime query failed            */
+
+/* Largest batch*head*n fused_mha_backward_noalloc accepts (8 MiB of scratch). */
+#define FUSED_MHA_NOALLOC_MAX_ROWS (1 << 20)
 
 /*
  * Element strides of a (batch, n, head, d) tensor whose last dimension is
@@ -123,6 +128,27 @@ int fused_mha_backward_strided(const void *query_ptr, const fused_mha_strides *q
                                const void *lse_ptr, void *workspace, size_t workspace_bytes,
                                void *d_query_ptr, void *d_key_ptr, void *d_value_ptr,
                                int batch, int head, int n, int d,
+                               float scale, int causal, void *stream);
+
+/*
+ * fused_mha_backward without a workspace argument and without any allocation:
+ * delta and lse*log2(e) go to a static device array inside the library
+ * (2 * FUSED_MHA_NOALLOC_MAX_ROWS floats = 8 MiB, held by every GPU the library
+ * runs on until the process ends).  No counterpart in the reference; it is for
+ * callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It calls no hipMalloc,
+ * hipFree or allocating library routine; the first call on a device looks up
+ * the array's device address, every later call only launches the kernels of
+ * fused_mha_backward.  Results are bit-identical to fused_mha_backward.
+ *   - batch*head*n above FUSED_MHA_NOALLOC_MAX_ROWS: FUSED_MHA_ERR_SCRATCH_LIMIT.
+ *   - The device that owns the tensors must be the current device.
+ *   - All calls on one GPU share that GPU's array: calls that overlap in time
+ *     on one GPU (two streams, two threads) race; serialise them.
+ */
+int fused_mha_backward_noalloc(const void *query_ptr, const void *key_ptr, const void *value_ptr,
+                               const void *output_ptr, const void *d_output_ptr, const void *lse_ptr,
+                               void *d_query_ptr, void *d_key_ptr, void *d_value_ptr,
+                               int batch, int head, int m, int n, int d,
                                float scale, int causal, void *stream);
 
 /*

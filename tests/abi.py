@@ -15,7 +15,8 @@ HEADER = os.path.join(ROOT, "include", "fused_mha.h")
 
 OK = 0
 (ERR_NULL_POINTER, ERR_BAD_SHAPE, ERR_BAD_HEAD_DIM, ERR_MISALIGNED, ERR_LAUNCH, ERR_BAD_SCALE, ERR_TOO_LARGE,
- ERR_BAD_STRIDE) = (-1, -2, -3, -4, -5, -6, -7, -8)
+ ERR_BAD_STRIDE, ERR_SCRATCH_LIMIT, ERR_RUNTIME) = (-1, -2, -3, -4, -5, -6, -7, -8, -9, -10)
+NOALLOC_MAX_ROWS = 1 << 20
 
 _vp, _i, _f, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
 
@@ -49,6 +50,8 @@ def load():
     lib.fused_mha_backward_workspace_bytes.restype = _sz
     lib.fused_mha_backward.argtypes = [_vp] * 7 + [_sz] + [_vp] * 3 + [_i] * 5 + [_f, _i, _vp]
     lib.fused_mha_backward.restype = _i
+    lib.fused_mha_backward_noalloc.argtypes = [_vp] * 9 + [_i] * 5 + [_f, _i, _vp]
+    lib.fused_mha_backward_noalloc.restype = _i
     lib.fused_mha_backward_delta.argtypes = [_vp, _vp, _vp, _vp, _sz] + [_i] * 4 + [_vp]
     lib.fused_mha_backward_delta.restype = _i
     lib.fused_mha_backward_dq.argtypes = [_vp] * 6 + [_sz, _vp] + [_i] * 4 + [_f, _i, _vp]
@@ -98,6 +101,18 @@ def backward(lib, q, k, v, out, dout, lse, scale, causal, stream=None, split=Fal
                                     dv.data_ptr(), B, H, N, N, D, scale, int(causal), s)
     assert rc == OK, lib.fused_mha_error_string(rc)
     return dq, dk, dv, ws.view(torch.float32)[:B * H * N].view(B, H, N)
+
+
+def backward_noalloc(lib, q, k, v, out, dout, lse, scale, causal, grads=None):
+    """fused_mha_backward_noalloc; `grads` = preallocated (dq, dk, dv) or None to allocate them here."""
+    B, N, H, D = q.shape
+    dq, dk, dv = grads if grads is not None else (torch.empty_like(q), torch.empty_like(q), torch.empty_like(q))
+    s = torch.cuda.current_stream().cuda_stream
+    rc = lib.fused_mha_backward_noalloc(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(),
+                                        lse.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, H, N, N, D,
+                                        scale, int(causal), s)
+    assert rc == OK, lib.fused_mha_error_string(rc)
+    return dq, dk, dv
 
 
 def forward_strided(lib, q, k, v, scale, causal):

@@ -19,7 +19,7 @@ def lib():
 def test_exports_every_declared_symbol(lib):
     names = abi.declared_symbols()
     assert names == sorted(["fused_mha_forward", "fused_mha_backward", "fused_mha_backward_workspace_bytes",
-                            "fused_mha_backward_delta", "fused_mha_backward_dq", "fused_mha_backward_dkdv",
+                            "fused_mha_backward_noalloc", "fused_mha_backward_delta", "fused_mha_backward_dq", "fused_mha_backward_dkdv",
                             "fused_mha_forward_strided", "fused_mha_backward_strided", "fused_mha_error_string"])
     for name in names:
         assert hasattr(lib, name), name
@@ -27,7 +27,7 @@ def test_exports_every_declared_symbol(lib):
 
 def test_error_strings(lib):
     seen = set()
-    for code in range(0, -9, -1):
+    for code in range(0, -11, -1):
         text = lib.fused_mha_error_string(code).decode()
         assert text and text not in seen
         seen.add(text)
@@ -73,6 +73,21 @@ def test_backward_validation_codes(lib):
     assert lib.fused_mha_backward_delta(p, None, p, p, ws, 1, 1, 32, 64, None) == abi.ERR_NULL_POINTER
     assert lib.fused_mha_backward_dq(p, p, p, p, p, p, ws, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
     assert lib.fused_mha_backward_dkdv(p, p, p, p, p, p, ws, p, None, 1, 1, 32, 64, 1.0, 0, None) == abi.ERR_NULL_POINTER
+
+
+def test_noalloc_validation_codes(lib):
+    """Rejected before the scratch address is looked up or anything is launched."""
+    p = 0x1000
+    g = lib.fused_mha_backward_noalloc
+    assert g(p, p, p, p, p, p, p, p, p, 1, 1, 40, 32, 64, 1.0, 0, None) == abi.ERR_BAD_SHAPE
+    assert g(p, p, p, p, p, p, p, p, p, 1, 1, 32, 32, 96, 1.0, 0, None) == abi.ERR_BAD_HEAD_DIM
+    rows = abi.NOALLOC_MAX_ROWS
+    assert g(p, p, p, p, p, p, p, p, p, 1, 2, rows // 2 + 1, rows // 2 + 1, 64, 1.0, 0, None) == abi.ERR_SCRATCH_LIMIT
+    assert g(p, p, p, p, p, p, p, p, p, 4, 64, 8192, 8192, 128, 1.0, 1, None) == abi.ERR_SCRATCH_LIMIT
+    assert b"NOALLOC_MAX_ROWS" in lib.fused_mha_error_string(abi.ERR_SCRATCH_LIMIT)
+    import re
+    text = open(abi.HEADER).read()
+    assert int(re.search(r"#define FUSED_MHA_NOALLOC_MAX_ROWS \(1 << (\d+)\)", text).group(1)) == 20
 
 
 def test_strided_validation_codes(lib):
