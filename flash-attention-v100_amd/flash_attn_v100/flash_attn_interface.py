@@ -1,3 +1,6 @@
+# The shape of this API (flash_attn_func over a torch.autograd.Function that calls
+# a compiled fwd/bwd pair) follows flash_attn_interface.py of FlashAttention,
+# Copyright (c) 2023, Tri Dao, through the reference's copy of that file.
 """Autograd front end, API-compatible with the reference's
 flash_attn_v100/flash_attn_interface.py:1-110.
 

@@ -10,7 +10,7 @@ import re
 import torch  # noqa: F401  (load order matters)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-LIB_PATH = os.path.join(ROOT, "flash-attention-v100_amd", "lib", "libfused_mha.so")
+LIB_PATH = os.path.join(ROOT, "flash-attention-v100_amd", "flash_attn_v100", "lib", "libfused_mha.so")
 HEADER = os.path.join(ROOT, "include", "fused_mha.h")
 
 OK = 0

@@ -213,3 +213,27 @@ int main() {
     exe = tmp_path / "check_block_map"
     subprocess.check_call(["g++", "-O1", "-std=c++17", "-I", inc, str(src), "-o", str(exe)])
     assert subprocess.check_output([str(exe)]).decode().strip() == "ok"
+
+
+def test_installed_distribution_imports_without_pythonpath(tmp_path):
+    """`pip install .` (the wheel `python setup.py install` / `pip wheel .` build; reference setup.py:151-172,
+    README.md:21-23) puts the package, the extension and the kernel library into one place, and the package
+    imports from there with no path into this tree."""
+    import os
+    import subprocess
+    import sys
+
+    pkg = os.path.join(abi.ROOT, "flash-attention-v100_amd")
+    target = tmp_path / "site"
+    subprocess.check_call([sys.executable, "-m", "pip", "install", "--no-deps", "--no-build-isolation", "--no-index",
+                           "--quiet", "--target", str(target), pkg])
+    assert (target / "flash_attn_v100_cuda.so").exists()
+    assert (target / "flash_attn_v100" / "lib" / "libfused_mha.so").exists()
+    code = ("import sys, os; sys.path.insert(0, %r); import flash_attn_v100, flash_attn_v100_cuda; "
+            "assert os.path.dirname(flash_attn_v100.__file__).startswith(%r); "
+            "assert flash_attn_v100_cuda.__file__.startswith(%r); "
+            "print(flash_attn_v100.__version__, callable(flash_attn_v100.flash_attn_func))") % (
+                str(target), str(target), str(target))
+    env = {k: v for k, v in os.environ.items() if k != "PYTHONPATH"}
+    out = subprocess.check_output([sys.executable, "-c", code], cwd=str(tmp_path), env=env).decode()
+    assert out.split() == ["0.0.1", "True"]
