@@ -18,11 +18,13 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (ROOT, os.path.join(ROOT, "flash-attention-v100_amd"), os.path.join(ROOT, "tests")):
+for _p in (ROOT, os.path.join(ROOT, "flash-attention-v100_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
 PEAK_TFLOPS = 2516.6  # MI355X dense fp16 MFMA, vendor figure
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, vendor figure
+SUSTAINED_LAUNCHES = 300
 
 CONFIGS = [  # name, B, H, N, D, causal
     ("plumbing_b1_h4_n128_d64", 1, 4, 128, 64, False),
@@ -37,6 +39,50 @@ HEADLINE = 3
 def fwd_flops(B, H, N, D, causal):
     f = 4.0 * B * H * N * N * D
     return f * 0.5 if causal else f
+
+
+def min_hbm_bytes(B, H, N, D):
+    """Algorithmic HBM bytes: forward reads q, k, v and writes o + lse; backward reads q, k, v, o, dO, lse
+    and writes dq, dk, dv."""
+    t = B * N * H * D * 2
+    stat = B * H * N * 4
+    return 4 * t + stat, 8 * t + stat
+
+
+def load_c_abi():
+    """ctypes binding of the entry points of include/fused_mha.h that the per-kernel timing uses."""
+    import ctypes
+    import torch  # noqa: F401  (first, so that the library binds to the HIP runtime torch loaded)
+
+    path = os.path.join(ROOT, "flash-attention-v100_amd", "flash_attn_v100", "lib", "libfused_mha.so")
+    if not os.path.exists(path):
+        sys.exit("bench.py: %s is not built (python setup.py build_ext --inplace in flash-attention-v100_amd/)" % path)
+    lib = ctypes.CDLL(path)
+    vp, i, f, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+    lib.fused_mha_forward.argtypes = [vp] * 5 + [i] * 5 + [f, i, vp]
+    lib.fused_mha_backward_workspace_bytes.argtypes = [i] * 4
+    lib.fused_mha_backward_workspace_bytes.restype = sz
+    lib.fused_mha_backward_delta.argtypes = [vp, vp, vp, vp, sz] + [i] * 4 + [vp]
+    lib.fused_mha_backward_dq.argtypes = [vp] * 6 + [sz, vp] + [i] * 4 + [f, i, vp]
+    lib.fused_mha_backward_dkdv.argtypes = [vp] * 6 + [sz, vp, vp] + [i] * 4 + [f, i, vp]
+    return lib
+
+
+def sustained_ms(fn, launches=SUSTAINED_LAUNCHES, warmup=10):
+    """Per-call device-event times of `launches` back-to-back calls; returns (median, list)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+    ev[0].record()
+    for n in range(launches):
+        fn()
+        ev[n + 1].record()
+    torch.cuda.synchronize()
+    ts = [ev[n].elapsed_time(ev[n + 1]) for n in range(launches)]
+    return sorted(ts)[launches // 2], ts
 
 
 def time_ms(fn, steps, warmup):
@@ -81,21 +127,24 @@ def bench_config(B, H, N, D, causal, steps, warmup):
         out.backward(do)
         q.grad = k.grad = v.grad = None
 
-    t_f = time_ms(fwd, steps, warmup)
-    t_fb = time_ms(fwd_bwd, steps, warmup)
+    t_f = sustained_ms(fwd, max(50, steps), max(10, warmup))[0]
+    t_fb = sustained_ms(fwd_bwd, max(50, steps), max(10, warmup))[0]
     ff = fwd_flops(B, H, N, D, causal)
-    return {"fwd_ms": t_f, "fwd_bwd_ms": t_fb, "fwd_tflops": ff / t_f / 1e9, "fwd_bwd_tflops": 3.5 * ff / t_fb / 1e9}
+    bytes_f, bytes_b = min_hbm_bytes(B, H, N, D)
+    return {"fwd_ms": t_f, "fwd_bwd_ms": t_fb, "fwd_tflops": ff / t_f / 1e9, "fwd_bwd_tflops": 3.5 * ff / t_fb / 1e9,
+            "fwd_hbm_frac": bytes_f / (t_f * 1e-3) / (PEAK_HBM_GBS * 1e9),
+            "fwd_bwd_hbm_frac": (bytes_f + bytes_b) / (t_fb * 1e-3) / (PEAK_HBM_GBS * 1e9)}
 
 
 def kernel_times(B, H, N, D, causal, steps, warmup):
     """Average duration of each kernel, timed one by one through the C ABI."""
     import torch
-    import abi
 
-    lib = abi.load()
+    lib = load_c_abi()
     q, k, v, do = make_device_inputs(B, H, N, D)
     scale = 1.0 / math.sqrt(D)
-    out, lse = abi.forward(lib, q, k, v, scale, causal)
+    out = torch.empty_like(q)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
     nbytes = lib.fused_mha_backward_workspace_bytes(B, H, N, D)
     ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
@@ -110,6 +159,10 @@ def kernel_times(B, H, N, D, causal, steps, warmup):
         "fmha_bwd_dkdv_kernel": lambda: lib.fused_mha_backward_dkdv(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes,
                                                                      p(dk), p(dv), B, H, N, D, scale, c, s),
     }
+    for name, fn in calls.items():  # each pass once, in dependency order, and every return code checked
+        rc = fn()
+        if rc != 0:
+            sys.exit("bench.py: %s returned %d" % (name, rc))
     return {name: time_ms(fn, steps, warmup) for name, fn in calls.items()}
 
 
@@ -119,13 +172,24 @@ def cpu_baseline(B, H, N, D, causal, budget_s=12.0):
     import torch
     from oracle import attention_oracle as ao
 
-    cores = os.cpu_count() or 1
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or 1 << 30)
     torch.set_num_threads(cores)
     g = torch.Generator(device="cpu")
     g.manual_seed(20)
     q, k, v, do = (torch.randn((1, N, 1, D), generator=g).half() for _ in range(4))
     scale = 1.0 / math.sqrt(D)
     ao.attention_forward(q[:, :256], k[:, :256], v[:, :256], scale, causal)  # warm the thread pool
+    others = {}
+    for cname, cB, cH, cN, cD, cc in CONFIGS[:HEADLINE]:  # the smaller configurations, whole: warm-up + median of 3
+        cq, ck, cv, cdo = (torch.randn((cB, cN, cH, cD), generator=g).half() for _ in range(4))
+        cs, times = 1.0 / math.sqrt(cD), []
+        for rep in range(4):
+            t0 = time.perf_counter()
+            ao.attention_forward(cq, ck, cv, cs, cc)
+            ao.attention_backward(cq, ck, cv, cdo, cs, cc)
+            times.append(time.perf_counter() - t0)
+        med = sorted(times[1:])[1]
+        others[cname] = {"seconds": round(med, 5), "tflops": round(3.5 * fwd_flops(cB, cH, cN, cD, cc) / med / 1e12, 5)}
     done, t0 = 0, time.perf_counter()
     while done < B * H:
         ao.attention_forward(q, k, v, scale, causal)
@@ -135,7 +199,7 @@ def cpu_baseline(B, H, N, D, causal, budget_s=12.0):
             break
     dt = time.perf_counter() - t0
     flops = 3.5 * fwd_flops(1, 1, N, D, causal) * done
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port", "other_configs": others,
             "sample": f"{done} of {B * H} (batch, head) slices of the headline workload, fwd+bwd, "
                       f"fp32 torch on {cores} threads, {dt:.1f} s; dense N^2 work done, causal-halved FLOPs counted"}
 
@@ -150,6 +214,9 @@ def main():
     ap.add_argument("--config-index", type=int, default=HEADLINE,
                     help="which entry of CONFIGS is the measured workload (default: the headline, %d); "
                          "other indices are for profiling the other configurations" % HEADLINE)
+    ap.add_argument("--launch-trace", metavar="FILE",
+                    help="write the duration of each of %d back-to-back forward launches to FILE "
+                         "(launch index, milliseconds)" % SUSTAINED_LAUNCHES)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times (reference point for HBM byte counters)")
     args = ap.parse_args()
@@ -200,6 +267,15 @@ def main():
     fwd_ms = time_ms(fwd_only, args.steps, args.warmup)
     fwd_tflops = ff / fwd_ms / 1e9
 
+    # sustained figures: median of per-call device-event times over many back-to-back calls
+    fwd_sus_ms, fwd_trace = sustained_ms(fwd_only)
+    step_sus_ms, _ = sustained_ms(step)
+    if args.launch_trace:
+        with open(args.launch_trace, "w") as fh:
+            fh.write("# launch index, forward duration in ms (%s, back to back after 10 warm-up launches)\n" % name)
+            for n, t in enumerate(fwd_trace):
+                fh.write("%d %.4f\n" % (n, t))
+
     # per-kernel durations and the roofline of the slowest kernel
     kt = kernel_times(B, H, N, D, causal, args.steps, args.warmup)
     # algorithmic FLOPs per launch: the GEMMs of the 5-GEMM backward / 2-GEMM forward
@@ -218,7 +294,7 @@ def main():
     others = {}
     if not args.headline_only:
         for cname, cB, cH, cN, cD, cc in CONFIGS:
-            r = bench_config(cB, cH, cN, cD, cc, max(5, args.steps // 2), max(3, args.warmup // 2))
+            r = bench_config(cB, cH, cN, cD, cc, args.steps, args.warmup)
             r["fwd_frac_peak"] = r["fwd_tflops"] / PEAK_TFLOPS
             r["fwd_bwd_frac_peak"] = r["fwd_bwd_tflops"] / PEAK_TFLOPS
             others[cname] = {key: round(val, 5) for key, val in r.items()}
@@ -232,6 +308,11 @@ def main():
         "config": {"workload": name, "batch": B, "heads": H, "seq_len": N, "head_dim": D, "causal": causal},
         "frac_of_peak": value / PEAK_TFLOPS,
         "fwd": {"ms": fwd_ms, "tflops": fwd_tflops, "frac_of_peak": fwd_tflops / PEAK_TFLOPS},
+        "value_sustained": {"launches": SUSTAINED_LAUNCHES, "ms_median": step_sus_ms,
+                            "tflops": 3.5 * ff / step_sus_ms / 1e9,
+                            "frac_of_peak": 3.5 * ff / step_sus_ms / 1e9 / PEAK_TFLOPS},
+        "fwd_sustained": {"launches": SUSTAINED_LAUNCHES, "ms_median": fwd_sus_ms, "tflops": ff / fwd_sus_ms / 1e9,
+                          "frac_of_peak": ff / fwd_sus_ms / 1e9 / PEAK_TFLOPS},
         "roofline": roofline,
         "all_configs": others,
     }
