@@ -85,14 +85,28 @@ __device__ __forceinline__ int acc_row(int rb, int r, int hh) {
   return rb * 32 + 8 * (r >> 2) + 4 * hh + (r & 3);
 }
 
-// Store a [D][32 resident] fp32 accumulator, scaled, as fp16 rows of a
-// (B, N, H, D) tensor.  Lane (i, hh) owns resident row `row`; per 32-feature
-// block it holds features 8*g + 4*hh + 0..3 for g = 0..3.
+// Store a [D][32 resident] fp32 accumulator, scaled, as fp16 rows of a dense
+// (B, N, H, D) tensor, through a staging tile in LDS that belongs to the wave
+// (32 rows of kStagePitch bytes): each lane first writes the 4-feature pieces it
+// holds of its own row, then the wave reads the tile back row-wise, so that
+// every row leaves as whole 16-byte pieces written by neighbouring lanes (a
+// 256-byte row by 16 lanes, as the reference's epilogue does with its 128-bit
+// stores, kernel/fused_mha_kernel.cu:318-322, 714-734).  Lane (i, hh) owns row
+// row0 + i; per 32-feature block it holds features 8*g + 4*hh + 0..3 for g = 0..3.
+// The caller makes sure (with a block barrier) that nobody still reads what the
+// staging tile overwrites.
 template <int D>
-__device__ __forceinline__ void store_resident(half_t* __restrict__ base, long row_stride, int row, int n,
-                                               const f16v (&acc)[TileGeom<D>::kDBlocks], float mul, int hh) {
-  if (row >= n) return;
-  half_t* p = base + (long)row * row_stride;
+struct StageGeom {
+  static constexpr int kPitch = D * 2 + 16;        // bytes per row: 16-byte aligned, rows on different banks
+  static constexpr int kBytes = kResident * kPitch;  // per wave
+};
+template <int D>
+__device__ __forceinline__ void store_resident(half_t* __restrict__ base, long row_stride, int row0, int n,
+                                               const f16v (&acc)[TileGeom<D>::kDBlocks], float mul, int lane,
+                                               char* __restrict__ stage) {
+  constexpr int kPitch = StageGeom<D>::kPitch;
+  const int i = lane & 31, hh = lane >> 5;
+  char* mine = stage + i * kPitch + hh * 8;
 #pragma unroll
   for (int db = 0; db < TileGeom<D>::kDBlocks; ++db) {
 #pragma unroll
@@ -100,8 +114,18 @@ __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long r
       h4 v;
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = (half_t)(acc[db][4 * g + e] * mul);
-      *reinterpret_cast<h4*>(p + db * 32 + 8 * g + 4 * hh) = v;
+      *reinterpret_cast<h4*>(mine + (db * 32 + 8 * g) * 2) = v;
     }
+  }
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the wave's own writes have landed
+  asm volatile("" ::: "memory");
+  constexpr int kLanesPerRow = D / 8, kRowsPerPass = 64 / kLanesPerRow;
+  const int r_in = lane / kLanesPerRow, ch = lane % kLanesPerRow;
+#pragma unroll
+  for (int pass = 0; pass < kResident / kRowsPerPass; ++pass) {
+    const int r = pass * kRowsPerPass + r_in;
+    const h8 v = *reinterpret_cast<const h8*>(stage + r * kPitch + ch * 16);
+    if (row0 + r < n) *reinterpret_cast<h8*>(base + (long)(row0 + r) * row_stride + ch * 8) = v;
   }
 }
 
@@ -475,7 +499,9 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
 
   const float l_tot = l_run + other_half(l_run);
   const float inv = 1.f / l_tot;
-  store_resident<D>(O + head_off, rs, qi, N, o, inv, hh);
+  static_assert(kFwdWaves * StageGeom<D>::kBytes <= 2 * kRing * T::kBytes, "the output staging tiles fit the rings");
+  block_barrier();  // every wave is done with the rings: they become the staging tiles
+  store_resident<D>(O + head_off, rs, q0w, N, o, inv, lane, smem + wave * StageGeom<D>::kBytes);
   if (hh == 0 && qi < N) LSE[((long)b * H + h) * N + qi] = (m_run * c + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }
 
@@ -719,6 +745,7 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
   };
 
   wait_vm<0>();  // resident rows, statistics and the first copies
+  f16v dq[G::kDBlocks];  // role B's accumulator
   if (!role_b) {
     for (int j = 0; j <= nt; ++j) {
       step_sync(j);
@@ -733,7 +760,6 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
       }
     }
   } else {
-    f16v dq[G::kDBlocks];
 #pragma unroll
     for (int db = 0; db < G::kDBlocks; ++db)
 #pragma unroll
@@ -775,8 +801,10 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
       }
       if (j < ntw) gemm1(v_ring + (j % 3) * T::kBytes, x, stat);
     }
-    store_resident<D>(dQ + head_off, rs, qi, N, dq, scale, hh);
   }
+  static_assert(kDqPairs * StageGeom<D>::kBytes <= 7 * T::kBytes, "the output staging tiles fit the rings");
+  block_barrier();  // every wave is done with the rings: they become the staging tiles
+  if (role_b) store_resident<D>(dQ + head_off, rs, q0w, N, dq, scale, lane, smem + pair * StageGeom<D>::kBytes);
 }
 
 // ---------------------------------------------------------------------------
@@ -1051,8 +1079,11 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
     }
   }
 
-  if (!role_b) store_resident<D>(dV + head_off, rs, ki, N, acc, 1.f, hh);
-  else store_resident<D>(dK + head_off, rs, ki, N, acc, scale, hh);
+  static_assert(kKvWaves * StageGeom<D>::kBytes <= 7 * T::kBytes, "the output staging tiles fit the rings");
+  block_barrier();  // every wave is done with the rings: they become the staging tiles
+  char* const stage = smem + wave * StageGeom<D>::kBytes;
+  if (!role_b) store_resident<D>(dV + head_off, rs, k0w, N, acc, 1.f, lane, stage);
+  else store_resident<D>(dK + head_off, rs, k0w, N, acc, scale, lane, stage);
 }
 
 // ---------------------------------------------------------------------------
