@@ -215,8 +215,10 @@ def main():
                     help="which entry of CONFIGS is the measured workload (default: the headline, %d); "
                          "other indices are for profiling the other configurations" % HEADLINE)
     ap.add_argument("--launch-trace", metavar="FILE",
-                    help="write the duration of each of %d back-to-back forward launches to FILE "
-                         "(launch index, milliseconds)" % SUSTAINED_LAUNCHES)
+                    help="write the duration of each back-to-back forward launch of a longer run to FILE "
+                         "(launch index, milliseconds since the first launch, duration in milliseconds)")
+    ap.add_argument("--launch-trace-count", type=int, default=6000,
+                    help="launches in the --launch-trace run (default 6000, about two seconds)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times (reference point for HBM byte counters)")
     args = ap.parse_args()
@@ -271,10 +273,16 @@ def main():
     fwd_sus_ms, fwd_trace = sustained_ms(fwd_only)
     step_sus_ms, _ = sustained_ms(step)
     if args.launch_trace:
+        torch.cuda.synchronize()
+        time.sleep(2.0)  # let the clocks settle back after the work above
+        _, long_trace = sustained_ms(fwd_only, args.launch_trace_count, 0)
         with open(args.launch_trace, "w") as fh:
-            fh.write("# launch index, forward duration in ms (%s, back to back after 10 warm-up launches)\n" % name)
-            for n, t in enumerate(fwd_trace):
-                fh.write("%d %.4f\n" % (n, t))
+            fh.write("# %s forward, %d launches back to back after 2 s of idle: launch index, ms since the first "
+                     "launch, duration in ms\n" % (name, len(long_trace)))
+            at = 0.0
+            for n, t in enumerate(long_trace):
+                fh.write("%d %.3f %.4f\n" % (n, at, t))
+                at += t
 
     # per-kernel durations and the roofline of the slowest kernel
     kt = kernel_times(B, H, N, D, causal, args.steps, args.warmup)
