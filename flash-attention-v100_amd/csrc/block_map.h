@@ -23,7 +23,7 @@
 // contiguous runs, one per XCD, so that each of those slices is shared by as
 // few XCDs as possible.
 #ifndef FMHA_SLICES_IN_FLIGHT
-#define FMHA_SLICES_IN_FLIGHT 4
+#define FMHA_SLICES_IN_FLIGHT 2
 #endif
 constexpr int kSlicesInFlight = FMHA_SLICES_IN_FLIGHT;
 FMHA_HOST_DEVICE void fmha_slice_and_block(int lin, int slices, int blocks_per_slice, int& slice,
