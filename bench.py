@@ -22,7 +22,8 @@ for _p in (ROOT, os.path.join(ROOT, "flash-attention-v100_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
-PEAK_TFLOPS = 2516.6  # MI355X dense fp16 MFMA, vendor figure
+PEAK_TFLOPS = 2516.6  # MI355X dense fp16 MFMA, vendor figure (256 CUs x 4 SIMDs x 1024 FLOP/clk at NOMINAL_MHZ)
+NOMINAL_MHZ = 2400
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, vendor figure
 SUSTAINED_LAUNCHES = 300
 
@@ -100,6 +101,93 @@ def time_ms(fn, steps, warmup):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / steps
+
+
+# The shader clock while a kernel runs.  rocm-smi is started by a helper process that was
+# itself started before this process touched the GPU (a process that has initialised the GPU
+# starts no programs); the helper waits for a line on its stdin, samples, and answers with one
+# JSON line.
+SAMPLER = r"""
+import json, re, subprocess, sys
+for line in sys.stdin:
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=30).stdout
+        m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", out)
+        print(json.dumps({"sclk_mhz": int(m.group(1)) if m else None}), flush=True)
+    except Exception as e:
+        print(json.dumps({"sclk_mhz": None, "error": str(e)}), flush=True)
+"""
+
+
+def start_clock_sampler():
+    import subprocess
+
+    try:
+        return subprocess.Popen([sys.executable, "-c", SAMPLER], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    except OSError:
+        return None
+
+
+def sclk_under_load(sampler, fn, settle_s=1.0, limit_s=40.0):
+    """Shader clock in MHz as rocm-smi reports it while fn() is launched back to back (None if it cannot be read)."""
+    import select
+    import torch
+
+    if sampler is None or sampler.poll() is not None:
+        return None
+    t0 = time.perf_counter()
+    asked = False
+    while time.perf_counter() - t0 < limit_s:
+        for _ in range(100):
+            fn()
+        torch.cuda.synchronize()
+        if not asked and time.perf_counter() - t0 > settle_s:
+            sampler.stdin.write("sample\n")
+            sampler.stdin.flush()
+            asked = True
+        if asked and select.select([sampler.stdout], [], [], 0)[0]:
+            try:
+                return json.loads(sampler.stdout.readline()).get("sclk_mhz")
+            except ValueError:
+                return None
+    return None
+
+
+def occupancy_sweep(path):
+    """Duration of the forward, dQ and dK/dV kernels of B1 N4096 D128 non-causal as the number of heads, and with
+    it the number of busy CUs, grows: every work group does the same work in every row of the table."""
+    import torch
+
+    lib = load_c_abi()
+    B, N, D = 1, 4096, 128
+    scale = 1.0 / math.sqrt(D)
+    with open(path, "w") as fh:
+        fh.write("# B1 N4096 D128 non-causal; medians of 100 launches, microseconds; 256 CUs; work groups per kernel:\n")
+        fh.write("# forward heads*16 (256 queries each), dQ and dK/dV heads*32 (128 rows each)\n")
+        fh.write("# heads fwd_groups fwd_us fwd_us_per_round dq_us dkdv_us\n")
+        for H in (2, 4, 8, 16, 32, 64):
+            q, k, v, do = make_device_inputs(B, H, N, D)
+            out = torch.empty_like(q)
+            lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+            nbytes = lib.fused_mha_backward_workspace_bytes(B, H, N, D)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+            dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
+            s = torch.cuda.current_stream().cuda_stream
+            p = lambda t: t.data_ptr()
+            calls = [
+                lambda: lib.fused_mha_forward(p(q), p(k), p(v), p(out), p(lse), B, H, N, N, D, scale, 0, s),
+                lambda: lib.fused_mha_backward_delta(p(out), p(do), p(lse), p(ws), nbytes, B, H, N, D, s),
+                lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dq), B, H, N, D, scale, 0, s),
+                lambda: lib.fused_mha_backward_dkdv(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dk), p(dv),
+                                                    B, H, N, D, scale, 0, s),
+            ]
+            for fn in calls:
+                if fn() != 0:
+                    sys.exit("bench.py: a kernel of the occupancy sweep failed")
+            us = [sustained_ms(fn, 100, 20)[0] * 1e3 for fn in (calls[0], calls[2], calls[3])]
+            groups = H * N // 256
+            rounds = max(1, -(-groups // 256))
+            fh.write("%d %d %.1f %.1f %.1f %.1f\n" % (H, groups, us[0], us[0] / rounds, us[1], us[2]))
 
 
 def make_device_inputs(B, H, N, D, seed=20):
@@ -219,11 +307,33 @@ def main():
                          "(launch index, milliseconds since the first launch, duration in milliseconds)")
     ap.add_argument("--launch-trace-count", type=int, default=6000,
                     help="launches in the --launch-trace run (default 6000, about two seconds)")
+    ap.add_argument("--microbench", metavar="FILE",
+                    help="first run the stand-alone programs of flash-attention-v100_amd/microbench/bin (instruction "
+                         "issue and MFMA rates, atomic-add throughput) and write what they print to FILE")
+    ap.add_argument("--occupancy-sweep", metavar="FILE",
+                    help="write kernel durations of B1 N4096 D128 for 2 .. 64 heads (32 .. 1024 forward work groups) to FILE")
+    ap.add_argument("--no-clock-sample", action="store_true", help="do not read the shader clock under load (rocm-smi)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times (reference point for HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus)
+
+    if args.microbench:  # child processes: started before this process touches the GPU
+        import subprocess
+
+        with open(args.microbench, "w") as fh:
+            for prog in ("issue_rate", "atomic_add"):
+                exe = os.path.join(ROOT, "flash-attention-v100_amd", "microbench", "bin", prog)
+                if not os.path.exists(exe):
+                    sys.exit("bench.py: %s is not built (python flash-attention-v100_amd/setup.py build_microbench)" % exe)
+                fh.write("== %s\n" % prog)
+                fh.flush()
+                subprocess.run([exe], stdout=fh, stderr=subprocess.STDOUT, timeout=120, check=True)
+
+    # (not under a profiler: its preloaded library has initialised the GPU before this program started)
+    profiled = "rocprof" in os.environ.get("LD_PRELOAD", "") or any(key.startswith("ROCPROF") for key in os.environ)
+    sampler = None if args.no_clock_sample or profiled else start_clock_sampler()  # before anything touches the GPU
 
     import torch
     from flash_attn_v100 import flash_attn_func
@@ -284,6 +394,19 @@ def main():
                 fh.write("%d %.3f %.4f\n" % (n, at, t))
                 at += t
 
+    if args.occupancy_sweep:
+        occupancy_sweep(args.occupancy_sweep)
+
+    # the shader clock the device runs at under these two loads (the published peak assumes NOMINAL_MHZ)
+    fwd_mhz = sclk_under_load(sampler, fwd_only)
+    step_mhz = sclk_under_load(sampler, step)
+    if sampler is not None:
+        sampler.stdin.close()
+    clock = {"nominal_mhz": NOMINAL_MHZ, "fwd_sclk_mhz": fwd_mhz, "step_sclk_mhz": step_mhz,
+             "source": "rocm-smi --showclocks, one sample after a second of back-to-back launches",
+             "peak_at_fwd_sclk_tflops": PEAK_TFLOPS * fwd_mhz / NOMINAL_MHZ if fwd_mhz else None,
+             "peak_at_step_sclk_tflops": PEAK_TFLOPS * step_mhz / NOMINAL_MHZ if step_mhz else None}
+
     # per-kernel durations and the roofline of the slowest kernel
     kt = kernel_times(B, H, N, D, causal, args.steps, args.warmup)
     # algorithmic FLOPs per launch: the GEMMs of the 5-GEMM backward / 2-GEMM forward
@@ -322,6 +445,7 @@ def main():
         "fwd_sustained": {"launches": SUSTAINED_LAUNCHES, "ms_median": fwd_sus_ms, "tflops": ff / fwd_sus_ms / 1e9,
                           "frac_of_peak": ff / fwd_sus_ms / 1e9 / PEAK_TFLOPS},
         "roofline": roofline,
+        "clock": clock,
         "all_configs": others,
     }
     if not args.no_cpu_baseline:
