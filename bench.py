@@ -103,19 +103,35 @@ def time_ms(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
-# The shader clock while a kernel runs.  rocm-smi is started by a helper process that was
-# itself started before this process touched the GPU (a process that has initialised the GPU
-# starts no programs); the helper waits for a line on its stdin, samples, and answers with one
-# JSON line.
+# The shader clock and the socket power while a kernel runs.  amd-smi (or rocm-smi) is started
+# by a helper process that was itself started before this process touched the GPU (a process that
+# has initialised the GPU starts no programs); the helper waits for a line on its stdin, samples,
+# and answers with one JSON line.
 SAMPLER = r"""
 import json, re, subprocess, sys
-for line in sys.stdin:
-    try:
-        out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=30).stdout
-        m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", out)
-        print(json.dumps({"sclk_mhz": int(m.group(1)) if m else None}), flush=True)
+def sample():
+    res = {"sclk_mhz": None, "socket_power_w": None, "xcd_mhz": None}
+    try:  # amd-smi: socket power and the clock of every XCD
+        out = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=30).stdout
+        m = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", out)
+        if m:
+            res["socket_power_w"] = int(m.group(1))
+        clk = [int(x) for x in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", out)]
+        if clk:
+            res["xcd_mhz"] = clk
+            res["sclk_mhz"] = round(sum(clk) / len(clk))
     except Exception as e:
-        print(json.dumps({"sclk_mhz": None, "error": str(e)}), flush=True)
+        res["amd_smi_error"] = str(e)
+    if res["sclk_mhz"] is None:
+        try:
+            out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=30).stdout
+            m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", out)
+            res["sclk_mhz"] = int(m.group(1)) if m else None
+        except Exception as e:
+            res["rocm_smi_error"] = str(e)
+    return res
+for line in sys.stdin:
+    print(json.dumps(sample()), flush=True)
 """
 
 
@@ -129,12 +145,14 @@ def start_clock_sampler():
 
 
 def sclk_under_load(sampler, fn, settle_s=1.0, limit_s=40.0):
-    """Shader clock in MHz as rocm-smi reports it while fn() is launched back to back (None if it cannot be read)."""
+    """One sample of the shader clock (MHz, mean over the XCDs) and the socket power (W) while fn() is launched
+    back to back; a dict of None values if they cannot be read."""
     import select
     import torch
 
+    nothing = {"sclk_mhz": None, "socket_power_w": None, "xcd_mhz": None}
     if sampler is None or sampler.poll() is not None:
-        return None
+        return nothing
     t0 = time.perf_counter()
     asked = False
     while time.perf_counter() - t0 < limit_s:
@@ -147,10 +165,10 @@ def sclk_under_load(sampler, fn, settle_s=1.0, limit_s=40.0):
             asked = True
         if asked and select.select([sampler.stdout], [], [], 0)[0]:
             try:
-                return json.loads(sampler.stdout.readline()).get("sclk_mhz")
+                return json.loads(sampler.stdout.readline())
             except ValueError:
-                return None
-    return None
+                return nothing
+    return nothing
 
 
 def occupancy_sweep(path):
@@ -398,12 +416,15 @@ def main():
         occupancy_sweep(args.occupancy_sweep)
 
     # the shader clock the device runs at under these two loads (the published peak assumes NOMINAL_MHZ)
-    fwd_mhz = sclk_under_load(sampler, fwd_only)
-    step_mhz = sclk_under_load(sampler, step)
+    fwd_load = sclk_under_load(sampler, fwd_only)
+    step_load = sclk_under_load(sampler, step)
     if sampler is not None:
         sampler.stdin.close()
+    fwd_mhz, step_mhz = fwd_load["sclk_mhz"], step_load["sclk_mhz"]
     clock = {"nominal_mhz": NOMINAL_MHZ, "fwd_sclk_mhz": fwd_mhz, "step_sclk_mhz": step_mhz,
-             "source": "rocm-smi --showclocks, one sample after a second of back-to-back launches",
+             "fwd_socket_power_w": fwd_load["socket_power_w"], "step_socket_power_w": step_load["socket_power_w"],
+             "fwd_xcd_mhz": fwd_load["xcd_mhz"],
+             "source": "amd-smi metric -p -c (else rocm-smi --showclocks), one sample after a second of back-to-back launches",
              "peak_at_fwd_sclk_tflops": PEAK_TFLOPS * fwd_mhz / NOMINAL_MHZ if fwd_mhz else None,
              "peak_at_step_sclk_tflops": PEAK_TFLOPS * step_mhz / NOMINAL_MHZ if step_mhz else None}
 
