@@ -104,42 +104,57 @@ def time_ms(fn, steps, warmup):
 
 
 # The shader clock and the socket power while a kernel runs.  amd-smi (or rocm-smi) is started
-# by a helper process that was itself started before this process touched the GPU (a process that
-# has initialised the GPU starts no programs); the helper waits for a line on its stdin, samples,
-# and answers with one JSON line.
-SAMPLER = r"""
-import json, re, subprocess, sys
-def sample():
+# by a helper process (this file run with --sampler) that was itself started before this process
+# touched the GPU: a process that has initialised the GPU starts no programs.  The helper waits
+# for a line on its stdin, samples, and answers with one JSON line.
+def parse_amd_smi(text):
+    """Socket power (W) and per-XCD shader clocks (MHz) from the text of `amd-smi metric -p -c`."""
+    import re
+
     res = {"sclk_mhz": None, "socket_power_w": None, "xcd_mhz": None}
-    try:  # amd-smi: socket power and the clock of every XCD
-        out = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=30).stdout
-        m = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", out)
-        if m:
-            res["socket_power_w"] = int(m.group(1))
-        clk = [int(x) for x in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", out)]
-        if clk:
-            res["xcd_mhz"] = clk
-            res["sclk_mhz"] = round(sum(clk) / len(clk))
-    except Exception as e:
-        res["amd_smi_error"] = str(e)
-    if res["sclk_mhz"] is None:
-        try:
-            out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=30).stdout
-            m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", out)
-            res["sclk_mhz"] = int(m.group(1)) if m else None
-        except Exception as e:
-            res["rocm_smi_error"] = str(e)
+    m = re.search(r"SOCKET_POWER:\s*(\d+)\s*W", text)
+    if m:
+        res["socket_power_w"] = int(m.group(1))
+    clk = [int(x) for x in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", text)]
+    if clk:
+        res["xcd_mhz"] = clk
+        res["sclk_mhz"] = round(sum(clk) / len(clk))
     return res
-for line in sys.stdin:
-    print(json.dumps(sample()), flush=True)
-"""
+
+
+def parse_rocm_smi(text):
+    """Shader clock (MHz) from the text of `rocm-smi --showclocks`, or None."""
+    import re
+
+    m = re.search(r"sclk clock level:\s*\d+:\s*\((\d+)Mhz\)", text)
+    return int(m.group(1)) if m else None
+
+
+def sampler_main():
+    import subprocess
+
+    for _ in sys.stdin:
+        res = {"sclk_mhz": None, "socket_power_w": None, "xcd_mhz": None}
+        try:
+            res = parse_amd_smi(subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True,
+                                               timeout=30).stdout)
+        except (OSError, subprocess.SubprocessError) as e:
+            res["amd_smi_error"] = str(e)
+        if res["sclk_mhz"] is None:
+            try:
+                res["sclk_mhz"] = parse_rocm_smi(subprocess.run(["rocm-smi", "--showclocks"], capture_output=True,
+                                                                text=True, timeout=30).stdout)
+            except (OSError, subprocess.SubprocessError) as e:
+                res["rocm_smi_error"] = str(e)
+        print(json.dumps(res), flush=True)
 
 
 def start_clock_sampler():
     import subprocess
 
     try:
-        return subprocess.Popen([sys.executable, "-c", SAMPLER], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+        return subprocess.Popen([sys.executable, os.path.abspath(__file__), "--sampler"], stdin=subprocess.PIPE,
+                                stdout=subprocess.PIPE, text=True)
     except OSError:
         return None
 
@@ -311,6 +326,8 @@ def cpu_baseline(B, H, N, D, causal, budget_s=12.0):
 
 
 def main():
+    if sys.argv[1:] == ["--sampler"]:
+        return sampler_main()
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)

@@ -4,11 +4,16 @@ launch, and the extension raises RuntimeError like the reference's TORCH_CHECKs
 (kernel/fused_mha_api.cpp:25-47).  No compute call is made here."""
 import ctypes
 import inspect
+import os
+import sys
 
 import pytest
 import torch
 
 import abi
+
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 @pytest.fixture(scope="module")
@@ -237,3 +242,53 @@ def test_installed_distribution_imports_without_pythonpath(tmp_path):
     env = {k: v for k, v in os.environ.items() if k != "PYTHONPATH"}
     out = subprocess.check_output([sys.executable, "-c", code], cwd=str(tmp_path), env=env).decode()
     assert out.split() == ["0.0.1", "True"]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py is a one-GPU benchmark: --gpus N with N > 1 exits with a message that says so."""
+    import subprocess
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr
+
+
+def test_bench_clock_sampler_helper():
+    """The helper bench.py starts for the clock and power sample: parsers on recorded tool output, and the
+    one-line-in, one-JSON-line-out protocol (on a machine without the tools the values are null)."""
+    import json
+    import subprocess
+
+    sys.path.insert(0, ROOT)
+    import bench
+
+    text = ("GPU: 0\n    POWER:\n        SOCKET_POWER: 1315 W\n        GFX_VOLTAGE: N/A\n    CLOCK:\n"
+            "        GFX_0:\n            CLK: 1885 MHz\n            MIN_CLK: 500 MHz\n            MAX_CLK: 2400 MHz\n"
+            "        GFX_1:\n            CLK: 1821 MHz\n            MIN_CLK: 500 MHz\n")
+    got = bench.parse_amd_smi(text)
+    assert got == {"sclk_mhz": 1853, "socket_power_w": 1315, "xcd_mhz": [1885, 1821]}
+    assert bench.parse_amd_smi("no such tool") == {"sclk_mhz": None, "socket_power_w": None, "xcd_mhz": None}
+    assert bench.parse_rocm_smi("GPU[0]\t\t: sclk clock level: 1: (1849Mhz)\n") == 1849
+    assert bench.parse_rocm_smi("") is None
+
+    p = bench.start_clock_sampler()
+    assert p is not None
+    p.stdin.write("sample\n")
+    p.stdin.flush()
+    reply = json.loads(p.stdout.readline())
+    assert set(("sclk_mhz", "socket_power_w", "xcd_mhz")) <= set(reply)
+    p.stdin.close()
+    assert p.wait(timeout=60) == 0
+
+
+def test_flop_and_byte_counts_of_the_bench():
+    sys.path.insert(0, ROOT)
+    import bench
+
+    assert bench.fwd_flops(2, 32, 4096, 128, True) == 4 * 2 * 32 * 4096 * 4096 * 128 / 2
+    assert bench.fwd_flops(16, 12, 512, 64, False) == 4 * 16 * 12 * 512 * 512 * 64
+    fwd_bytes, bwd_bytes = bench.min_hbm_bytes(2, 32, 4096, 128)
+    tensor = 2 * 32 * 4096 * 128 * 2
+    assert fwd_bytes == 4 * tensor + 2 * 32 * 4096 * 4  # q, k, v, o and lse
+    assert bwd_bytes >= 8 * tensor  # q, k, v, o, dO in; dq, dk, dv out
