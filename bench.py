@@ -330,8 +330,10 @@ def main():
         return sampler_main()
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=30)
-    ap.add_argument("--warmup", type=int, default=10)
+    # defaults: the power management needs 20-30 ms of load after an idle period before the launch
+    # durations settle, so the warm-up covers that (40 steps are about 50 ms)
+    ap.add_argument("--steps", type=int, default=60)
+    ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true")
     ap.add_argument("--config-index", type=int, default=HEADLINE,
