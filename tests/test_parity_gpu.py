@@ -220,6 +220,33 @@ def test_non_dense_inputs_and_side_stream():
     assert _err(qg.grad, dq_ref) <= G_TOL and _err(kg.grad, dk_ref) <= G_TOL and _err(vg.grad, dv_ref) <= G_TOL
 
 
+def test_random_shapes_and_scales(lib):
+    """Forty shapes drawn from a fixed seed: batch 1-3, 1-12 heads (slice counts that are and are not
+    multiples of 8), lengths 1-1500 (tiny, ragged, whole tiles), both head sizes, both mask modes, four
+    scales including a negative one and one that makes the softmax peaky.  The outputs are fp16, so the
+    tolerance grows with the magnitude of the expected tensor (half an ulp of fp16 at 8 is 4e-3)."""
+    import random
+
+    rng = random.Random(2024)
+    torch.set_num_threads(16)
+    for case in range(40):
+        B, H, D = rng.randint(1, 3), rng.choice([1, 2, 3, 5, 7, 8, 9, 12]), rng.choice([64, 128])
+        N = rng.choice([rng.randint(1, 70), rng.randint(60, 400), rng.randint(400, 1500), 64 * rng.randint(1, 20)])
+        causal = rng.random() < 0.6
+        scale = rng.choice([1 / math.sqrt(D), 0.1, -0.07, 0.3])
+        print(f"case {case}: B{B} H{H} N{N} D{D} causal={causal} scale={scale:.3f}", flush=True)
+        q, k, v, do = ao.make_inputs(B, N, H, D, seed=case)
+        qg, kg, vg, dog = (t.cuda() for t in (q, k, v, do))
+        out, lse = abi.forward(lib, qg, kg, vg, scale, causal)
+        dq, dk, dv, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal)
+        torch.cuda.synchronize()
+        o_ref, lse_ref = ao.attention_forward(q, k, v, scale, causal)
+        refs = (o_ref,) + tuple(ao.attention_backward(q, k, v, do, scale, causal))
+        assert (lse.cpu() - lse_ref).abs().max().item() <= LSE_TOL
+        for name, got, want, tol in zip(("O", "dQ", "dK", "dV"), (out, dq, dk, dv), refs, (O_TOL, G_TOL, G_TOL, G_TOL)):
+            assert _err(got, want) <= tol * max(1.0, want.abs().max().item()), (case, name)
+
+
 @pytest.mark.parametrize("D,causal", [(64, True), (128, False), (128, True)])
 def test_wide_score_ranges(lib, D, causal):
     """Scores whose running maximum keeps growing along the keys and rows dominated by
