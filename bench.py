@@ -460,6 +460,8 @@ def main():
         traffic = json.load(open(tpath)).get(dominant)
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_TFLOPS, "traffic": traffic,
+                # the same against the peak at the shader clock measured under the fwd+bwd load (informative)
+                "frac_at_step_sclk": achieved / clock["peak_at_step_sclk_tflops"] if clock["peak_at_step_sclk_tflops"] else None,
                 "kernel_ms": kt, "peak_check_tflops": peak_check}
 
     others = {}
