@@ -37,6 +37,12 @@
 
 #include "fused_mha.h"
 #include "block_map.h"
+#ifndef DS_NT_LOAD
+#define DS_NT_LOAD 1
+#endif
+#ifndef DS_NT_STORE
+#define DS_NT_STORE 1
+#endif
 
 // Backward workspace of fused_mha_backward_noalloc (delta and lse*log2(e), fp32
 // (batch, head, n) each): lives in the code object, one copy per GPU, so that
@@ -107,9 +113,11 @@ struct StageGeom {
 template <int D>
 __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long row_stride, int row0, int n,
                                                const f16v (&acc)[TileGeom<D>::kDBlocks], float mul, int lane,
-                                               char* __restrict__ stage) {
+                                               char* __restrict__ stage, int my_row = -1) {
+  // my_row: the row (0..31, relative to row0) this lane's column of the accumulator belongs
+  // to, when that is not lane & 31 (see fmha_bwd_dq_spill_kernel)
   constexpr int kPitch = StageGeom<D>::kPitch;
-  const int i = lane & 31, hh = lane >> 5;
+  const int i = my_row < 0 ? (lane & 31) : my_row, hh = lane >> 5;
   char* mine = stage + i * kPitch + hh * 8;
 #pragma unroll
   for (int db = 0; db < TileGeom<D>::kDBlocks; ++db) {
@@ -192,6 +200,25 @@ __device__ __forceinline__ void copy16(const half_t* tile_base, int voff, char* 
       : "v"(voff), "s"(tile_base), "s"(lds_addr)
       : "memory");
 }
+// The same for data that is read once (the non-temporal hint keeps it from displacing
+// the tiles other work groups re-read out of the L2).
+__device__ __forceinline__ void copy16_stream(const half_t* tile_base, int voff, char* lds_block) {
+  const unsigned lds_addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds_block;
+  unsigned saved_m0;
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %3\n\t"
+      "s_nop 0\n\t"
+#if DS_NT_LOAD
+      "global_load_lds_dwordx4 %1, %2 nt\n\t"
+#else
+      "global_load_lds_dwordx4 %1, %2\n\t"
+#endif
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0)
+      : "v"(voff), "s"(tile_base), "s"(lds_addr)
+      : "memory");
+}
 
 // The same with 4 bytes per lane (256 bytes per instruction): lane l fetches the
 // dword at base + voff and it lands in LDS at lds_dst + 4 * l.
@@ -247,14 +274,24 @@ __device__ __forceinline__ h8 swz_cols(const char* tile, int c16, int db, const 
 // builtin (not inline asm) so that the compiler's wait-count bookkeeping sees it.
 template <int N>
 __device__ __forceinline__ void wait_vm() {
-  static_assert(N >= 0 && N < 16, "vmcnt immediate");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+  static_assert(N >= 0 && N < 64, "vmcnt immediate");  // bits 3:0 and 15:14 of the immediate
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 __device__ __forceinline__ void block_barrier() {
   __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads have landed
   asm volatile("" ::: "memory");       // keep LDS accesses on their side of the barrier
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+// Wait until at most min(later, kMax) * kPer of this wave's copies are in flight.
+template <int kPer, int kMax>
+__device__ __forceinline__ void wait_vm_tiles(int later) {
+  if constexpr (kMax == 0) {
+    wait_vm<0>();
+  } else {
+    if (later >= kMax) wait_vm<kMax * kPer>();
+    else wait_vm_tiles<kPer, kMax - 1>(later);
+  }
 }
 template <int V>
 struct IntTag { static constexpr int value = V; };
@@ -835,12 +872,25 @@ constexpr int kKvWaves = 2 * kKvPairs;
 constexpr int kKvThreads = kKvWaves * 64;
 constexpr int kKvBlockKeys = kKvPairs * kResident;
 
-template <int D, bool CAUSAL>
+//
+// SPILL: wave B also writes every dS tile it forms (fp16, without the scale factor) to
+// the workspace `dS`, for fmha_bwd_dq_spill_kernel, which then needs no S and dP of
+// its own.  Layout per (batch, head) slice, np = n rounded up to 128:
+//   [np / 128 query blocks][np / 64 key tiles] x 16 KiB, the tile a block of 128 queries
+//   streams per 64 keys, made of 16 pieces of 1 KiB:
+//   [2 halves of 32 keys][2 query tiles of 64][4 chunks of 16 queries] x 1 KiB.
+// A 1 KiB piece is what one store instruction of wave B writes: lane l = 32 * hh + i
+// (key i, half hh) puts the 16 bytes of registers it holds for the chunk at 16 * l
+// (consecutive lanes, consecutive addresses); inside a chunk position 8*hh + e holds
+// query 8*(e >> 2) + 4*hh + (e & 3).  Rows of keys at or past n are written as zeros; (key tile, query
+// tile) pairs above the diagonal are not written (and not read) under causal masking.
+template <int D, bool CAUSAL, bool SPILL>
 __global__ void __launch_bounds__(kKvThreads, 1)
 fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
                      const half_t* __restrict__ dO, Strides qs, Strides ks, Strides vs, Strides gs,
                      const float* __restrict__ delta, const float* __restrict__ lse2,
-                     half_t* __restrict__ dK, half_t* __restrict__ dV, int H, int N, int nnb, float c, float scale) {
+                     half_t* __restrict__ dK, half_t* __restrict__ dV, half_t* __restrict__ dS, int np, int H, int N,
+                     int nnb, float c, float scale) {
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kKvWaves;  // copies per wave per tile, per tensor
@@ -1006,7 +1056,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 
   // Per iteration: wait for tile `it` (issued two iterations ago; the copies of tile
   // it+1 may still be in flight), one barrier, issue the copies of tile it+2.
-  auto step_sync = [&](int it) __attribute__((always_inline)) {
+  auto step_wait = [&](int it) __attribute__((always_inline)) {
     if (it + 1 < n_it) {
       if (wave == 0) wait_vm<2 * kIPW + 2>();
       else wait_vm<2 * kIPW>();
@@ -1014,8 +1064,16 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
       wait_vm<0>();
     }
     block_barrier();
+  };
+  auto step_sync = [&](int it) __attribute__((always_inline)) {
+    step_wait(it);
     if (it + 2 < n_it) copy_tiles(it + 2);
   };
+  // where this lane's registers of dS go (SPILL): its key's 32 bytes in chunk 0 of query tile 0 of
+  // query block 0; per query tile t: + (t >> 1) * np * 128 + (t & 1) * 2048, per chunk + 512 (elements)
+  half_t* const ds_lane = SPILL ? dS + ((long)bh * (np >> 7)) * np * 128 + (long)(k0w >> 6) * 8192 +
+                                      ((k0w >> 5) & 1) * 4096 + lane * 8
+                                : nullptr;
   wait_vm<0>();  // resident rows and the first copies: nothing is left for the compiler to wait on in the loops
   if (!role_b) {
     for (int it = 0; it <= n_it; ++it) {
@@ -1051,11 +1109,15 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
       for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
     for (int it = 0; it <= n_it; ++it) {
-      step_sync(it);
-      if (it >= 1 && tile_active(it - 1)) {  // the part that needs P, one tile behind
-        const char* Ql = q_ring + ((it - 1) & 3) * T::kBytes;
+      // SPILL: the stores of dS are issued before this iteration's tile copies, so that the
+      // wait at the top of the next iteration (everything but the newest copies) covers them
+      // whatever order stores and copies complete in.
+      if (SPILL) step_wait(it);
+      else step_sync(it);
+      const bool prev_active = it >= 1 && tile_active(it - 1);
+      h8 y[4];
+      if (prev_active) {  // the part that needs P, one tile behind
         const char* pr = p_mine + ((it - 1) & 1) * kPBytes;
-        h8 y[4];
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
           const h8 p0 = *reinterpret_cast<const h8*>(pr + rb * 2048);
@@ -1066,8 +1128,27 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
             y[rb * 2 + 1][e] = (half_t)(-(float)p1[e] * x[rb][8 + e]);
           }
         }
-        gemm2(Ql, y);
+        if (SPILL) {
+          if (k0w + kResident > N && ki >= N) {  // keys past the end contribute nothing to dQ
+#pragma unroll
+            for (int c16 = 0; c16 < 4; ++c16)
+#pragma unroll
+              for (int e = 0; e < 8; ++e) y[c16][e] = (half_t)0.f;
+          }
+          const int t = t_begin + it - 1;  // the query tile
+          half_t* dst = ds_lane + (long)(t >> 1) * np * 128 + (t & 1) * 2048;
+#pragma unroll
+          for (int c16 = 0; c16 < 4; ++c16) {
+#if DS_NT_STORE
+            __builtin_nontemporal_store(y[c16], reinterpret_cast<h8*>(dst + c16 * 512));
+#else
+            *reinterpret_cast<h8*>(dst + c16 * 512) = y[c16];
+#endif
+          }
+        }
       }
+      if (SPILL && it + 2 < n_it) copy_tiles(it + 2);
+      if (prev_active) gemm2(q_ring + ((it - 1) & 3) * T::kBytes, y);
       if (it < n_it && tile_active(it)) {
         const char* Gl = g_ring + (it % 3) * T::kBytes;
         const char* Sl = st_ring + (it % 3) * kStBytes + st_off;
@@ -1090,6 +1171,183 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
   char* const stage = smem + wave * StageGeom<D>::kBytes;
   if (!role_b) store_resident<D>(dV + head_off, rs, k0w, N, acc, 1.f, lane, stage);
   else store_resident<D>(dK + head_off, rs, k0w, N, acc, scale, lane, stage);
+}
+
+// ---------------------------------------------------------------------------
+// Backward, dQ from spilled dS: dQ = scale * dS K, one GEMM, for callers whose
+// workspace holds the dS tiles fmha_bwd_dkdv_kernel<.., SPILL> wrote (layout there).
+// Block = 128 queries, 8 waves; wave w owns the 32 queries qb = w & 3 of the block
+// and half of the features (w >> 2), and computes per 64 keys
+//     dQ^T[d][q] += K^T[d][key] dS^T[key][q]
+// with both operands read transposed out of LDS (the K tile as everywhere else, the
+// dS tile as its 1 KiB pieces of [32 keys][16 queries]), so the order of the keys
+// inside a 16-key step is the same for both.
+// The kernel is bound by reading dS from HBM once, so what matters is the number of
+// bytes in flight: the 16 KiB dS tiles go through a 6-slot ring, five tiles ahead,
+// copied by waves 0-3 only; the K tiles (L2 hits) through a 3-slot ring, two ahead,
+// copied by waves 4-7 only.  A wave's copies complete in order, so a wave that issued
+// both would have to wait for young dS copies whenever it needs an older K tile.
+// The queries of a chunk sit in the order the dK/dV pass's registers held them (bits
+// 2 and 3 of the position inside 16 swapped); the epilogue puts the rows back in place.
+// (formula: reference kernel/fused_mha_kernel.cu:680-683.)
+// ---------------------------------------------------------------------------
+constexpr int kDsWaves = 8;
+constexpr int kDsThreads = kDsWaves * 64;
+constexpr int kDsBlockQ = 128;
+#ifndef DQS_RING_S
+#define DQS_RING_S 6
+#define DQS_RING_K 3
+#define DQS_OCC 1
+#endif
+constexpr int kDsRingS = DQS_RING_S;   // dS tiles
+constexpr int kDsRingK = DQS_RING_K;   // K tiles
+constexpr int kDsTileBytes = kTile * kDsBlockQ * 2;
+
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(kDsThreads, DQS_OCC)
+fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t* __restrict__ dS, int np,
+                         half_t* __restrict__ dQ, int H, int N, int nqb, float scale) {
+  using T = SwzTile<D>;             // K tile: 64 keys x D features
+  constexpr int kCopyWaves = kDsWaves / 2;
+  constexpr int kKIPW = T::kInstrs / kCopyWaves;           // K copies per K-copying wave and tile
+  constexpr int kSIPW = (kDsTileBytes / 1024) / kCopyWaves;  // dS copies per dS-copying wave and tile
+  constexpr int kDBW = D / 64;      // 32-feature blocks per wave
+  __shared__ __attribute__((aligned(1024))) char smem[kDsRingS * kDsTileBytes + kDsRingK * T::kBytes];
+  char* const s_ring = smem;
+  char* const k_ring = smem + kDsRingS * kDsTileBytes;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int qb = wave & 3, dh = wave >> 2;
+  const bool copies_k = wave >= kCopyWaves;
+  const int cw = wave & (kCopyWaves - 1);
+  const int i = lane & 31;
+  int bh, mb;
+  slice_and_block(nqb, bh, mb);
+  const int mblk = CAUSAL ? nqb - 1 - mb : mb;  // heavy blocks first
+  const int b = bh / H, h = bh - b * H;
+  const int rs = H * D;  // dQ is dense
+  const long head_off = ((long)b * N * H + h) * D;
+  const half_t* Kb = K + b * ks.b + (long)h * ks.h;
+  const half_t* Sb = dS + (((long)bh * nqb + mblk) * np) * kDsBlockQ;  // this block's np / 64 tiles of 16 KiB
+
+  const int nt_all = (N + kTile - 1) / kTile;
+  const int nt = CAUSAL ? min(nt_all, 2 * mblk + 2) : nt_all;  // tiles the block streams
+  const int qt = 2 * mblk + (qb >> 1);                         // this wave's query tile
+  const int jend = qt >= nt_all ? 0 : (CAUSAL ? min(nt, qt + 1) : nt);  // tiles this wave takes part in
+
+  // K copies: this wave's share of a tile (as in the other kernels).  dS copies: piece p = cw * kSIPW + u of
+  // the tile, 1 KiB, lane l fetching 16 bytes.  In memory a piece is [2 halves][32 keys] x 16 bytes; in LDS it
+  // becomes [32 keys][2 halves] x 16 bytes (rows of 16 queries), and the pieces of odd query chunks land rotated
+  // by 128 bytes (LDS offset o holds row-major byte (o - 128) mod 1024), which keeps the two halves of a 32-lane
+  // transposing read on different banks.
+  int c_row[kKIPW], c_kgoff[kKIPW], c_kblk[kKIPW];
+#pragma unroll
+  for (int u = 0; u < kKIPW; ++u) {
+    const int t = cw * kKIPW + u;
+    copy_src<D>(t, lane, ks.n, c_row[u], c_kgoff[u]);
+    c_kblk[u] = t * 1024;
+  }
+  int c_sgoff[kSIPW];
+#pragma unroll
+  for (int u = 0; u < kSIPW; ++u) {
+    const int piece = cw * kSIPW + u;
+    const int at = (piece & 1) ? (lane - 8) & 63 : lane;  // position (key, half) = (at >> 1, at & 1) of the piece in LDS
+    c_sgoff[u] = piece * 1024 + ((at & 1) * 32 + (at >> 1)) * 16;
+  }
+  auto copy_s = [&](int j, int slot) __attribute__((always_inline)) {
+    const half_t* sp = Sb + (long)j * (kDsTileBytes / 2);  // wave-uniform
+    char* dst = s_ring + slot * kDsTileBytes + cw * kSIPW * 1024;
+#pragma unroll
+    for (int u = 0; u < kSIPW; ++u) copy16_stream(sp, c_sgoff[u], dst + u * 1024);
+  };
+  auto copy_k = [&](int j, int slot) __attribute__((always_inline)) {
+    const int row0 = j * kTile;
+    const half_t* kp = Kb + (long)row0 * ks.n;  // wave-uniform
+    char* dst = k_ring + slot * T::kBytes;
+    if (row0 + kTile <= N) {
+#pragma unroll
+      for (int u = 0; u < kKIPW; ++u) copy16(kp, c_kgoff[u], dst + c_kblk[u]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < kKIPW; ++u) {  // rows past the end re-read row N-1 (their dS rows are zero)
+        const int back = max(row0 + c_row[u] - (N - 1), 0);
+        copy16(kp, c_kgoff[u] - back * ks.n * 2, dst + c_kblk[u]);
+      }
+    }
+  };
+  constexpr int kAheadS = kDsRingS - 1, kAheadK = kDsRingK - 1;
+  if (copies_k) {
+    for (int j = 0; j < kAheadK && j < nt; ++j) copy_k(j, j);
+  } else {
+    for (int j = 0; j < kAheadS && j < nt; ++j) copy_s(j, j);
+  }
+
+  // LDS offsets of this lane's transposing reads.  K tile: as in the other kernels.  dS tile: key step kc,
+  // read e: key row (kc & 1) * 16 + 8 * e + 4 * hhk + (L >> 2) of the piece [(kc >> 1)][query tile][chunk
+  // 2 * (qb & 1) + lane bit 4], 8 bytes at (L & 3) * 8 of its 32-byte row, plus the rotation of odd chunks.
+  int c_off[2];
+  swz_cols_off<D>(lane, c_off);
+  int s_off[2][2];
+  {
+    const int L = lane & 15, odd = (lane >> 4) & 1, hhk = lane >> 5;
+#pragma unroll
+    for (int kcl = 0; kcl < 2; ++kcl)
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int in_piece = (kcl * 16 + 8 * e + 4 * hhk + (L >> 2)) * 32 + (L & 3) * 8;
+        s_off[kcl][e] = ((qb >> 1) * 4 + 2 * (qb & 1) + odd) * 1024 + ((in_piece + odd * 128) & 1023);
+      }
+  }
+  auto s_frag = [&](const char* tile, int kc) __attribute__((always_inline)) {
+    typedef __attribute__((address_space(3))) s4 lds_s4;
+    const char* p = tile + (kc >> 1) * 8192;
+    s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + s_off[kc & 1][0]));
+    s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p + s_off[kc & 1][1]));
+    return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+
+  f16v acc[kDBW];
+#pragma unroll
+  for (int db = 0; db < kDBW; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+
+  int slot_s = 0, slot_k = 0;                        // ring slots of tile j
+  int next_s = kAheadS % kDsRingS, next_k = kAheadK % kDsRingK;  // ring slots of the tiles to copy next
+  for (int j = 0; j < nt; ++j) {
+    // tile j must have landed; the copies of the tiles after it (at most kAhead - 1 of them) may be in flight
+    const int later = nt - 1 - j;
+    if (copies_k) wait_vm_tiles<kKIPW, kAheadK - 1>(later);
+    else wait_vm_tiles<kSIPW, kAheadS - 1>(later);
+    block_barrier();  // tile j is visible to all; everybody is done with tile j - 1, whose slots are reused now
+    if (copies_k) {
+      if (j + kAheadK < nt) copy_k(j + kAheadK, next_k);
+    } else {
+      if (j + kAheadS < nt) copy_s(j + kAheadS, next_s);
+    }
+    if (j < jend) {
+      const char* Kl = k_ring + slot_k * T::kBytes;
+      const char* Sl = s_ring + slot_s * kDsTileBytes;
+#pragma unroll
+      for (int c16 = 0; c16 < 4; ++c16) {
+        const h8 bfrag = s_frag(Sl, c16);
+#pragma unroll
+        for (int db = 0; db < kDBW; ++db)
+          acc[db] = mfma(swz_cols<D>(Kl, c16, dh * kDBW + db, c_off), bfrag, acc[db]);
+      }
+    }
+    slot_s = slot_s + 1 == kDsRingS ? 0 : slot_s + 1;
+    slot_k = slot_k + 1 == kDsRingK ? 0 : slot_k + 1;
+    next_s = next_s + 1 == kDsRingS ? 0 : next_s + 1;
+    next_k = next_k + 1 == kDsRingK ? 0 : next_k + 1;
+  }
+  static_assert(kDsWaves * StageGeom<D / 2>::kBytes <= kDsRingS * kDsTileBytes, "the output staging tiles fit the ring");
+  block_barrier();  // every wave is done with the rings: they become the staging tiles
+  // column i of the accumulator is the query at position i of the wave's 32: bits 2 and 3 swapped
+  const int my_row = (i & 0x13) | ((i & 8) >> 1) | ((i & 4) << 1);
+  store_resident<D / 2>(dQ + head_off + dh * (D / 2), rs, mblk * kDsBlockQ + qb * kResident, N, acc, scale, lane,
+                        smem + wave * StageGeom<D / 2>::kBytes, my_row);
 }
 
 // ---------------------------------------------------------------------------
@@ -1171,13 +1429,26 @@ int dispatch_forward(const void* q, const fused_mha_strides* q_st, const void* k
 
 enum BwdPass { kPassDelta = 1, kPassDq = 2, kPassDkDv = 4, kPassAll = 7 };
 
+// Workspace of the backward: delta and lse * log2(e), fp32 (batch, head, n) each; then, for
+// the spill path, at the next multiple of 256 bytes, the fp16 dS tiles
+// (batch * head slices of np * np elements, np = n rounded up to 128).
+size_t stats_bytes(int batch, int head, int n) { return 2 * (size_t)batch * head * n * sizeof(float); }
+size_t spill_offset(int batch, int head, int n) { return (stats_bytes(batch, head, n) + 255) & ~(size_t)255; }
+int padded_n(int n) { return (n + 127) & ~127; }
+size_t spill_bytes(int batch, int head, int n) {
+  const size_t np = (size_t)padded_n(n);
+  return (size_t)batch * head * np * np * sizeof(half_t);
+}
+
 template <int D, bool CAUSAL>
-int launch_backward(int passes, const void* q, const void* k, const void* v, const void* o, const void* d_o,
-                    Strides qs, Strides ks, Strides vs, Strides gs, const void* lse, float* delta, void* dq, void* dk,
-                    void* dv, int batch, int head, int n, float scale, hipStream_t stream) {
-  // With all three passes asked for, the dQ pass produces delta and lse2 itself.
-  const bool dq_makes_stats = (passes & kPassAll) == kPassAll;
+int launch_backward(int passes, bool spill, const void* q, const void* k, const void* v, const void* o,
+                    const void* d_o, Strides qs, Strides ks, Strides vs, Strides gs, const void* lse, float* delta,
+                    void* dq, void* dk, void* dv, int batch, int head, int n, float scale, hipStream_t stream) {
+  // Without the spill and with all three passes asked for, the dQ pass produces delta and lse2 itself.
+  const bool dq_makes_stats = !spill && (passes & kPassAll) == kPassAll;
   float* lse2 = delta + (long)batch * head * n;
+  half_t* ds = spill ? (half_t*)((char*)delta + spill_offset(batch, head, n)) : nullptr;
+  const int np = padded_n(n);
   if ((passes & kPassDelta) && !dq_makes_stats) {
     const long rows = (long)batch * n * head;
     const long threads = rows * (D / 8);
@@ -1186,20 +1457,32 @@ int launch_backward(int passes, const void* q, const void* k, const void* v, con
       return FUSED_MHA_ERR_LAUNCH;
   }
   const float c = scale * kLog2e;
-  if (passes & kPassDq) {
+  auto dq_pass = [&]() {
+    if (spill) {
+      const int nqb = np / kDsBlockQ;
+      return launch(fmha_bwd_dq_spill_kernel<D, CAUSAL>, (unsigned)nqb * batch * head, kDsThreads, stream,
+                    (const half_t*)k, ks, (const half_t*)ds, np, (half_t*)dq, head, n, nqb, scale);
+    }
     const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;
     auto kernel = dq_makes_stats ? fmha_bwd_dq_kernel<D, CAUSAL, true> : fmha_bwd_dq_kernel<D, CAUSAL, false>;
-    if (launch(kernel, (unsigned)nmb * batch * head, kDqThreads, stream, (const half_t*)q, (const half_t*)k,
-               (const half_t*)v, (const half_t*)o, (const half_t*)d_o, qs, ks, vs, gs, (const float*)lse, delta, lse2,
-               (half_t*)dq, head, n, nmb, c, scale) != hipSuccess)
-      return FUSED_MHA_ERR_LAUNCH;
-  }
-  if (passes & kPassDkDv) {
+    return launch(kernel, (unsigned)nmb * batch * head, kDqThreads, stream, (const half_t*)q, (const half_t*)k,
+                  (const half_t*)v, (const half_t*)o, (const half_t*)d_o, qs, ks, vs, gs, (const float*)lse, delta, lse2,
+                  (half_t*)dq, head, n, nmb, c, scale);
+  };
+  auto dkdv_pass = [&]() {
     const int nnb = (n + kKvBlockKeys - 1) / kKvBlockKeys;
-    if (launch(fmha_bwd_dkdv_kernel<D, CAUSAL>, (unsigned)nnb * batch * head, kKvThreads, stream, (const half_t*)q,
-               (const half_t*)k, (const half_t*)v, (const half_t*)d_o, qs, ks, vs, gs, (const float*)delta,
-               (const float*)lse2, (half_t*)dk, (half_t*)dv, head, n, nnb, c, scale) != hipSuccess)
-      return FUSED_MHA_ERR_LAUNCH;
+    auto kernel = spill ? fmha_bwd_dkdv_kernel<D, CAUSAL, true> : fmha_bwd_dkdv_kernel<D, CAUSAL, false>;
+    return launch(kernel, (unsigned)nnb * batch * head, kKvThreads, stream, (const half_t*)q, (const half_t*)k,
+                  (const half_t*)v, (const half_t*)d_o, qs, ks, vs, gs, (const float*)delta, (const float*)lse2,
+                  (half_t*)dk, (half_t*)dv, ds, np, head, n, nnb, c, scale);
+  };
+  // The spilling dK/dV pass feeds the dQ pass; otherwise the dQ pass (which may make the statistics) goes first.
+  if (spill) {
+    if ((passes & kPassDkDv) && dkdv_pass() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+    if ((passes & kPassDq) && dq_pass() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+  } else {
+    if ((passes & kPassDq) && dq_pass() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
+    if ((passes & kPassDkDv) && dkdv_pass() != hipSuccess) return FUSED_MHA_ERR_LAUNCH;
   }
   return FUSED_MHA_OK;
 }
@@ -1215,7 +1498,10 @@ int dispatch_backward(int passes, const void* q, const fused_mha_strides* q_st, 
     return FUSED_MHA_ERR_NULL_POINTER;
   if (int rc = check_shape(batch, head, m, n, d)) return rc;
   if (!isfinite(scale)) return FUSED_MHA_ERR_BAD_SCALE;
-  if (workspace_bytes < 2 * (size_t)batch * head * n * sizeof(float)) return FUSED_MHA_ERR_BAD_SHAPE;
+  if (workspace_bytes < stats_bytes(batch, head, n)) return FUSED_MHA_ERR_BAD_SHAPE;
+  // A workspace with room for the dS tiles selects the spill path (5 GEMMs executed instead of 7).
+  const bool spill = spill_bytes(batch, head, n) <= FUSED_MHA_SPILL_MAX_BYTES &&
+                     workspace_bytes >= spill_offset(batch, head, n) + spill_bytes(batch, head, n);
   if (misaligned(q) || misaligned(k) || misaligned(v) || misaligned(o) || misaligned(d_o) || misaligned(lse) ||
       misaligned(workspace) || misaligned(dq) || misaligned(dk) || misaligned(dv))
     return FUSED_MHA_ERR_MISALIGNED;
@@ -1225,7 +1511,8 @@ int dispatch_backward(int passes, const void* q, const fused_mha_strides* q_st, 
   const Strides qs = to_strides(q_st, head, n, d), ks = to_strides(k_st, head, n, d),
                 vs = to_strides(v_st, head, n, d), gs = to_strides(g_st, head, n, d);
 #define FMHA_BWD(DD, CC) \
-  launch_backward<DD, CC>(passes, q, k, v, o, d_o, qs, ks, vs, gs, lse, delta, dq, dk, dv, batch, head, n, scale, s)
+  launch_backward<DD, CC>(passes, spill, q, k, v, o, d_o, qs, ks, vs, gs, lse, delta, dq, dk, dv, batch, head, n, \
+                          scale, s)
   if (d == 128) return causal ? FMHA_BWD(128, true) : FMHA_BWD(128, false);
   return causal ? FMHA_BWD(64, true) : FMHA_BWD(64, false);
 #undef FMHA_BWD
@@ -1268,9 +1555,15 @@ int fused_mha_forward_strided(const void* query_ptr, const fused_mha_strides* qu
                           lse_ptr, batch, head, n, n, d, scale, causal, stream);
 }
 
+size_t fused_mha_backward_min_workspace_bytes(int batch, int head, int n, int d) {
+  if (check_shape(batch, head, n, n, d) != FUSED_MHA_OK) return 0;
+  return stats_bytes(batch, head, n);
+}
+
 size_t fused_mha_backward_workspace_bytes(int batch, int head, int n, int d) {
   if (check_shape(batch, head, n, n, d) != FUSED_MHA_OK) return 0;
-  return 2 * (size_t)batch * head * n * sizeof(float);  // delta and lse * log2(e), fp32 (batch, head, n) each
+  if (spill_bytes(batch, head, n) > FUSED_MHA_SPILL_MAX_BYTES) return stats_bytes(batch, head, n);
+  return spill_offset(batch, head, n) + spill_bytes(batch, head, n);
 }
 
 int fused_mha_backward(const void* query_ptr, const void* key_ptr, const void* value_ptr, const void* output_ptr,

@@ -91,14 +91,28 @@ int fused_mha_forward_strided(const void *query_ptr, const fused_mha_strides *qu
                               int batch, int head, int n, int d,
                               float scale, int causal, void *stream);
 
+/* Largest dS spill (bytes) the backward will use; beyond it the recompute path runs. */
+#define FUSED_MHA_SPILL_MAX_BYTES ((size_t)16 << 30)
+
 /*
- * Bytes of device scratch fused_mha_backward needs for this problem size
- * (holds delta = rowsum(d_o * o) and lse * log2(e), both fp32 of shape
- * (batch, head, n), delta first).
- * Returns 0 for an invalid shape.  No counterpart in the reference, which
- * receives delta from Python (flash_attn_interface.py:43-44).
+ * Bytes of device scratch the backward works best with for this problem size.
+ * The workspace starts with delta = rowsum(d_o * o) and lse * log2(e), both
+ * fp32 of shape (batch, head, n), delta first: that much
+ * (fused_mha_backward_min_workspace_bytes) is always needed.  When the
+ * workspace also has room for the fp16 dS tiles (batch * head * np * np
+ * elements, np = n rounded up to 128; at most FUSED_MHA_SPILL_MAX_BYTES), the
+ * dK/dV pass writes the dS it forms there and the dQ pass is a single GEMM over
+ * them: five GEMMs are executed, as in the reference's one-pass backward
+ * (kernel/fused_mha_kernel.cu:564-713), instead of seven.  With the minimum
+ * workspace the dQ pass recomputes S and dP.  Both paths are deterministic and
+ * give the same dK and dV bits; dQ differs by summation order only.
+ * fused_mha_backward_workspace_bytes returns the larger size when the spill is
+ * within the limit, else the minimum; any size in between selects the
+ * recompute path.  Both return 0 for an invalid shape.  No counterpart in the
+ * reference, which receives delta from Python (flash_attn_interface.py:43-44).
  */
 size_t fused_mha_backward_workspace_bytes(int batch, int head, int n, int d);
+size_t fused_mha_backward_min_workspace_bytes(int batch, int head, int n, int d);
 
 /*
  * Backward: d_q, d_k, d_v of the forward above, given d_o, the forward's
@@ -153,15 +167,18 @@ int fused_mha_backward_noalloc(const void *query_ptr, const void *key_ptr, const
 
 /*
  * The three passes fused_mha_backward enqueues, one entry point each, so a
- * caller can time them separately or put the dQ pass and the dK/dV pass (which
- * are independent of each other, both depend on the delta pass) on different
- * streams.  Same conventions and workspace as fused_mha_backward.  No
+ * caller can time them separately or, with the minimum workspace, put the dQ
+ * pass and the dK/dV pass (then independent of each other, both depend on the
+ * delta pass) on different streams.  Same conventions and workspace as fused_mha_backward.  No
  * counterpart in the reference, whose backward is a single kernel
  * (kernel/fused_mha_kernel.cu:904-916).
  *   delta : workspace[b][h][i] = sum_j d_o[b][i][h][j] * o[b][i][h][j]  (fp32),
  *           followed by lse * log2(e) in the same shape
  *   dq    : d_q, streaming key/value tiles per block of 128 queries
  *   dkdv  : d_k and d_v, streaming query/d_o tiles per block of 128 keys
+ * With a workspace of fused_mha_backward_workspace_bytes (room for the dS
+ * tiles) the dkdv pass also writes dS and the dq pass reads it: dq must then
+ * run after dkdv, on the same workspace.
  */
 int fused_mha_backward_delta(const void *output_ptr, const void *d_output_ptr, const void *lse_ptr,
                              void *workspace, size_t workspace_bytes,

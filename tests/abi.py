@@ -48,6 +48,8 @@ def load():
     lib.fused_mha_forward.restype = _i
     lib.fused_mha_backward_workspace_bytes.argtypes = [_i] * 4
     lib.fused_mha_backward_workspace_bytes.restype = _sz
+    lib.fused_mha_backward_min_workspace_bytes.argtypes = [_i] * 4
+    lib.fused_mha_backward_min_workspace_bytes.restype = _sz
     lib.fused_mha_backward.argtypes = [_vp] * 7 + [_sz] + [_vp] * 3 + [_i] * 5 + [_f, _i, _vp]
     lib.fused_mha_backward.restype = _i
     lib.fused_mha_backward_noalloc.argtypes = [_vp] * 9 + [_i] * 5 + [_f, _i, _vp]
@@ -80,9 +82,12 @@ def forward(lib, q, k, v, scale, causal, stream=None):
     return out, lse
 
 
-def backward(lib, q, k, v, out, dout, lse, scale, causal, stream=None, split=False):
+def backward(lib, q, k, v, out, dout, lse, scale, causal, stream=None, split=False, min_workspace=False):
+    """min_workspace: pass only delta + lse2 (the dQ pass then recomputes S and dP) instead of the
+    workspace with room for the dS tiles (the dK/dV pass spills dS, the dQ pass is one GEMM)."""
     B, N, H, D = q.shape
-    nbytes = lib.fused_mha_backward_workspace_bytes(B, H, N, D)
+    nbytes = (lib.fused_mha_backward_min_workspace_bytes if min_workspace else
+              lib.fused_mha_backward_workspace_bytes)(B, H, N, D)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
     s = torch.cuda.current_stream().cuda_stream if stream is None else stream

@@ -24,6 +24,7 @@ def lib():
 def test_exports_every_declared_symbol(lib):
     names = abi.declared_symbols()
     assert names == sorted(["fused_mha_forward", "fused_mha_backward", "fused_mha_backward_workspace_bytes",
+                            "fused_mha_backward_min_workspace_bytes",
                             "fused_mha_backward_noalloc", "fused_mha_backward_delta", "fused_mha_backward_dq", "fused_mha_backward_dkdv",
                             "fused_mha_forward_strided", "fused_mha_backward_strided", "fused_mha_error_string"])
     for name in names:
@@ -40,11 +41,21 @@ def test_error_strings(lib):
 
 
 def test_workspace_bytes(lib):
-    assert lib.fused_mha_backward_workspace_bytes(2, 32, 4096, 128) == 2 * 2 * 32 * 4096 * 4
-    assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 64) == 2 * 4 * 128 * 4
-    assert lib.fused_mha_backward_workspace_bytes(1, 4, 100, 64) == 2 * 4 * 100 * 4  # any n > 0 is accepted
-    assert lib.fused_mha_backward_workspace_bytes(1, 4, 0, 64) == 0
-    assert lib.fused_mha_backward_workspace_bytes(1, 4, 128, 96) == 0
+    small = lib.fused_mha_backward_min_workspace_bytes
+    assert small(2, 32, 4096, 128) == 2 * 2 * 32 * 4096 * 4
+    assert small(1, 4, 128, 64) == 2 * 4 * 128 * 4
+    assert small(1, 4, 100, 64) == 2 * 4 * 100 * 4  # any n > 0 is accepted
+    assert small(1, 4, 0, 64) == 0
+    assert small(1, 4, 128, 96) == 0
+    # the preferred workspace adds room for the fp16 dS tiles: slices * np * np elements, np = n rounded up to
+    # 128, behind the statistics rounded up to 256 bytes
+    big = lib.fused_mha_backward_workspace_bytes
+    assert big(2, 32, 4096, 128) == 2 * 2 * 32 * 4096 * 4 + 64 * 4096 * 4096 * 2
+    assert big(1, 4, 100, 64) == 3328 + 4 * 128 * 128 * 2  # 3200 bytes of statistics -> 3328
+    assert big(1, 4, 0, 64) == 0 and big(1, 4, 128, 96) == 0
+    # past the spill limit (16 GiB) only the statistics are asked for
+    assert big(1, 32, 16384, 128) == small(1, 32, 16384, 128) + 32 * 16384 * 16384 * 2  # 16 GiB: still spilled
+    assert big(1, 64, 16384, 128) == small(1, 64, 16384, 128)                           # 32 GiB: recompute path
 
 
 def test_forward_validation_codes(lib):
