@@ -37,12 +37,6 @@
 
 #include "fused_mha.h"
 #include "block_map.h"
-#ifndef DS_NT_LOAD
-#define DS_NT_LOAD 1
-#endif
-#ifndef DS_NT_STORE
-#define DS_NT_STORE 1
-#endif
 
 // Backward workspace of fused_mha_backward_noalloc (delta and lse*log2(e), fp32
 // (batch, head, n) each): lives in the code object, one copy per GPU, so that
@@ -147,6 +141,26 @@ __device__ __forceinline__ void slice_and_block(int blocks_per_slice, int& slice
   fmha_slice_and_block(blockIdx.x, gridDim.x / blocks_per_slice, blocks_per_slice, slice, blk);
 }
 
+// Blocks of a persistent work group.  The launch's blocks are numbered as by
+// fmha_slice_and_block (heaviest first inside every XCD's groups of slices); work group w of G
+// takes, in round r, block r * G + w for even r and r * G + (w mirrored inside its XCD) for odd r.
+// Both keep the block number congruent to w modulo 8, i.e. on w's XCD, and the alternation pairs
+// the heavy blocks of one round with the light blocks of the next.  G is a multiple of 8 unless
+// the launch has a single round.
+struct PersistentBlocks {
+  int total;
+  __device__ __forceinline__ int lin(int r) const {  // >= total: this group has no block in round r
+    const int G = gridDim.x, w = blockIdx.x;
+    const int p = (r & 1) ? (((G >> 3) - 1 - (w >> 3)) << 3) + (w & 7) : w;
+    return r * G + p;
+  }
+  __device__ __forceinline__ int next_round(int r) const {  // the next round with a block for this group, or -1
+    for (++r; (long)r * gridDim.x < total; ++r)
+      if (lin(r) < total) return r;
+    return -1;
+  }
+};
+
 // ---------------------------------------------------------------------------
 // 64-row tiles copied global -> LDS by global_load_lds_dwordx4 (no registers in
 // between).  One wave-level instruction moves 1 KiB: 16 rows x 64 bytes, every
@@ -209,11 +223,7 @@ __device__ __forceinline__ void copy16_stream(const half_t* tile_base, int voff,
       "s_mov_b32 %0, m0\n\t"
       "s_mov_b32 m0, %3\n\t"
       "s_nop 0\n\t"
-#if DS_NT_LOAD
       "global_load_lds_dwordx4 %1, %2 nt\n\t"
-#else
-      "global_load_lds_dwordx4 %1, %2\n\t"
-#endif
       "s_mov_b32 m0, %0"
       : "=&s"(saved_m0)
       : "v"(voff), "s"(tile_base), "s"(lds_addr)
@@ -326,45 +336,57 @@ constexpr int kFwdThreads = kFwdWaves * 64;
 constexpr int kFwdBlockQ = kFwdWaves * kResident;
 constexpr int kRing = 3;
 
+// The kernel is persistent: the launch has one work group per CU (fewer for small
+// problems) and each walks its own list of blocks (PersistentBlocks).  While a block's
+// last tiles are being worked on, the first K and V tiles of the group's next block are
+// already copied into the ring slots that come next, and the next block's Q rows are
+// loaded during the last iteration (which no longer needs Q); O leaves through staging
+// tiles of its own in LDS.  So a block boundary costs one pipeline fill, not a work-group
+// launch, a round trip to HBM and an epilogue during which the CU has nothing else to do.
 template <int D, bool CAUSAL>
 __global__ void __launch_bounds__(kFwdThreads, 1)
 fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
                 Strides qs, Strides ks, Strides vs, half_t* __restrict__ O, float* __restrict__ LSE, int H, int N,
-                int nmb, float c, int negate_q) {
+                int nmb, int total, float c, int negate_q) {
   using G = TileGeom<D>;
   using T = SwzTile<D>;
   constexpr int kIPW = T::kInstrs / kFwdWaves;  // copy instructions per wave per tile
-  // K ring then V ring, kRing slots each.  The copies into the ring are inline
-  // asm (see copy16), so slots can be addressed at run time.
-  __shared__ __attribute__((aligned(1024))) char smem[2 * kRing * T::kBytes];
+  // K ring then V ring, kRing slots each, then per wave a staging tile for 64 features of
+  // its 32 output rows.  The copies into the ring are inline asm (see copy16), so slots
+  // can be addressed at run time.
+  __shared__ __attribute__((aligned(1024))) char smem[2 * kRing * T::kBytes + kFwdWaves * StageGeom<64>::kBytes];
   char* const k_ring = smem;
   char* const v_ring = smem + kRing * T::kBytes;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 31, hh = lane >> 5;
-  int bh, mb;
-  slice_and_block(nmb, bh, mb);
-  const int mblk = CAUSAL ? nmb - 1 - mb : mb;  // heavy blocks first
-  const int b = bh / H, h = bh - b * H;
+  char* const stage = smem + 2 * kRing * T::kBytes + wave * StageGeom<64>::kBytes;
   const int rs = H * D;  // O is dense
-  const long head_off = ((long)b * N * H + h) * D;
-  const half_t* Qb = Q + b * qs.b + (long)h * qs.h;
-  const half_t* Kb = K + b * ks.b + (long)h * ks.h;
-  const half_t* Vb = V + b * vs.b + (long)h * vs.h;
+  const int nt_all = (N + kTile - 1) / kTile;
+  const PersistentBlocks pb{total};
+  const int slices = total / nmb;
 
-  const int m0 = mblk * kFwdBlockQ;
-  const int q0w = m0 + wave * kResident;
-  const int qi = q0w + i;
-
-  // nt: tiles the block streams; ntw: tiles this wave has unmasked keys in.
-  int nt = (N + kTile - 1) / kTile;
-  int ntw = nt;
-  if (CAUSAL) {
-    nt = min(nt, (min(m0 + kFwdBlockQ, N) - 1) / kTile + 1);
-    ntw = min(nt, (min(q0w + kResident, N) - 1) / kTile + 1);
-    if (q0w >= N) ntw = 0;
-  }
+  struct Block {
+    const half_t *q, *k, *v;  // first row of the (batch, head) slice
+    long o_off, stat_off;     // of the slice in O and in LSE
+    int m0, nt;               // first query of the block; tiles it streams
+  };
+  auto decode = [&](int lin) __attribute__((always_inline)) {
+    int bh, mb;
+    fmha_slice_and_block(lin, slices, nmb, bh, mb);
+    const int mblk = CAUSAL ? nmb - 1 - mb : mb;  // heavy blocks first
+    const int b = bh / H, h = bh - b * H;
+    Block B;
+    B.q = Q + b * qs.b + (long)h * qs.h;
+    B.k = K + b * ks.b + (long)h * ks.h;
+    B.v = V + b * vs.b + (long)h * vs.h;
+    B.o_off = ((long)b * N * H + h) * D;
+    B.stat_off = ((long)b * H + h) * N;
+    B.m0 = mblk * kFwdBlockQ;
+    B.nt = CAUSAL ? min(nt_all, (min(B.m0 + kFwdBlockQ, N) - 1) / kTile + 1) : nt_all;
+    return B;
+  };
 
   // this wave's share of every tile copy
   int c_row[kIPW], c_kgoff[kIPW], c_vgoff[kIPW], c_blk[kIPW];
@@ -391,53 +413,49 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
     }
   };
 
-  copy_tile(Kb, ks.n, c_kgoff, k_ring, 0);
-  if (nt > 1) copy_tile(Kb, ks.n, c_kgoff, k_ring + T::kBytes, 1);
-  copy_tile(Vb, vs.n, c_vgoff, v_ring, 0);
-
   h8 qf[G::kKSteps];
-  {
-    const half_t* qp = Qb + (long)min(qi, N - 1) * qs.n + hh * 8;
+  auto load_q = [&](const Block& B) __attribute__((always_inline)) {
+    const half_t* qp = B.q + (long)min(B.m0 + wave * kResident + i, N - 1) * qs.n + hh * 8;
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) {
-      qf[kk] = *reinterpret_cast<const h8*>(qp + kk * 16);
-      if (negate_q) qf[kk] = -qf[kk];
-    }
-  }
+    for (int kk = 0; kk < G::kKSteps; ++kk) qf[kk] = *reinterpret_cast<const h8*>(qp + kk * 16);
+  };
 
   int k_off[2], v_off[2];
   swz_rows_off<D>(lane, k_off);
   swz_cols_off<D>(lane, v_off);
 
+  // state of the block being worked on
+  int q0w = 0, qi = 0, ntw = 0;
   f16v o[G::kDBlocks];
-#pragma unroll
-  for (int db = 0; db < G::kDBlocks; ++db)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
   f16v s[2];   // scores of the tile in flight
   h8 pf[4];    // its probabilities, fp16, B-operand order
 
+  // The fragment reads of both GEMMs run kLead MFMAs ahead of their use.  The order is written out
+  // and pinned with scheduling barriers: left to itself the scheduler, once registers get scarce,
+  // puts every read right before its MFMA, which then waits a full LDS round trip each time.
+  constexpr int kLead = 4;
   auto scores = [&](const char* Kl, int t) __attribute__((always_inline)) {
     if (t >= ntw) return;
+    constexpr int kN = 2 * G::kKSteps;  // MFMA n: key block rb = n & 1, feature step kk = n >> 1
+    h8 frag[kLead];
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int n = 0; n < kLead; ++n) frag[n] = swz_rows<D>(Kl, n & 1, n >> 1, k_off);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[rb][r] = 0.f;
+    for (int n = 0; n < kN; ++n) {
+      const int rb = n & 1, kk = n >> 1;
+      if (kk == 0) {
+        f16v zero;
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) {
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(swz_rows<D>(Kl, rb, kk, k_off), qf[kk], s[rb]);
+        for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+        s[rb] = mfma(frag[n % kLead], qf[kk], zero);
+      } else {
+        s[rb] = mfma(frag[n % kLead], qf[kk], s[rb]);
+      }
+      if (n + kLead < kN) frag[n % kLead] = swz_rows<D>(Kl, (n + kLead) & 1, (n + kLead) >> 1, k_off);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    // LDS reads run kLead MFMAs ahead of their use.
-    constexpr int kN = 2 * G::kKSteps, kLead = 4;
-    __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
-#pragma unroll
-    for (int n = 0; n < kN - kLead; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
   auto softmax = [&](int t) __attribute__((always_inline)) {
     if (t < 0 || t >= ntw) return;
@@ -487,65 +505,167 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   };
   auto accumulate = [&](const char* Vl, int t) __attribute__((always_inline)) {
     if (t < 0 || t >= ntw) return;
+    constexpr int kDB = G::kDBlocks, kN = 4 * kDB;  // MFMA n: key chunk c16 = n / kDB, feature block db = n % kDB
+    h8 frag[kLead];
 #pragma unroll
-    for (int c16 = 0; c16 < 4; ++c16) {
+    for (int n = 0; n < kLead; ++n) frag[n] = swz_cols<D>(Vl, n / kDB, n % kDB, v_off);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(swz_cols<D>(Vl, c16, db, v_off), pf[c16], o[db]);
+    for (int n = 0; n < kN; ++n) {
+      o[n % kDB] = mfma(frag[n % kLead], pf[n / kDB], o[n % kDB]);
+      if (n + kLead < kN) frag[n % kLead] = swz_cols<D>(Vl, (n + kLead) / kDB, (n + kLead) % kDB, v_off);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    // LDS reads (two per MFMA) run kLead MFMAs ahead of their use.
-    constexpr int kN = 4 * G::kDBlocks, kLead = 4;
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead, 0);
-#pragma unroll
-    for (int n = 0; n < kN - kLead; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
 
   const bool first_group = wave < kFwdWaves / 2;
-  // Everything issued so far (Q rows, first copies) is waited for here, once,
-  // so that no wait for a register load is left to be placed inside the loop,
-  // where it would also wait for the copies in flight.
-  wait_vm<0>();
-  // Iteration j: K(j) sits in K slot j % 3, V(j-1) in V slot (j-1) % 3; K(j+2)
-  // is copied into K slot (j+2) % 3 and V(j+1) into V slot (j+1) % 3.
+  // Iteration j of a block: K(j) sits in K slot s0, V(j-1) in V slot s2; K(j+2) is copied
+  // into K slot s2 and V(j+1) into V slot s1, where tiles past the block's last one are the
+  // first tiles of the group's next block (at most K(0), K(1) and V(0) of it).  The slots
+  // rotate after every iteration but a block's last, so the next block finds its tile 0 in s0.
   auto run = [&](auto group_tag) __attribute__((always_inline)) {
     constexpr bool kFirst = decltype(group_tag)::value == 0;
-    int s0 = 0, s1 = 1, s2 = 2;  // j % 3, (j+1) % 3, (j+2) % 3
-    for (int j = 0; j <= nt; ++j) {
-      // K(j) and V(j-1) were issued two iterations ago; what the previous
-      // iteration issued (K(j+1), V(j)) may still be in flight.
-      if (j + 1 < nt) wait_vm<2 * kIPW>();
-      else if (j < nt) wait_vm<kIPW>();
-      else wait_vm<0>();
-      block_barrier();
-      if (j + 2 < nt) copy_tile(Kb, ks.n, c_kgoff, k_ring + s2 * T::kBytes, j + 2);
-      if (j + 1 < nt) copy_tile(Vb, vs.n, c_vgoff, v_ring + s1 * T::kBytes, j + 1);
-      const char* Kl = k_ring + s0 * T::kBytes;
-      const char* Vl = v_ring + s2 * T::kBytes;
-      if (kFirst) {
-        accumulate(Vl, j - 1);
-        if (j < nt) { scores(Kl, j); softmax(j); }
-      } else {
-        softmax(j - 1);
-        accumulate(Vl, j - 1);
-        if (j < nt) scores(Kl, j);
+    int lin_cur = pb.lin(0), round = 0;
+    {
+      const Block first = decode(lin_cur);
+      copy_tile(first.k, ks.n, c_kgoff, k_ring, 0);
+      if (first.nt > 1) copy_tile(first.k, ks.n, c_kgoff, k_ring + T::kBytes, 1);
+      copy_tile(first.v, vs.n, c_vgoff, v_ring, 0);
+      load_q(first);
+    }
+    int s0 = 0, s1 = 1, s2 = 2;
+    // Copies this wave issued in the previous iteration: all it may leave in flight at the top of
+    // an iteration (the tiles needed now were issued earlier).  0 at a block's first iteration:
+    // everything issued so far (Q rows, the previous block's output rows) is waited for there, so
+    // that no wait for a register load is left to be placed inside the loop, where it would also
+    // wait for the copies in flight.
+    int in_flight = 0;
+    for (;;) {
+      // Only what the main loop needs is decoded here; the next block and the output addresses are
+      // worked out after it, so that they do not occupy scalar registers across it.
+      const half_t *cur_k, *cur_v;
+      int nt;
+      {
+        const Block cur = decode(lin_cur);
+        cur_k = cur.k;
+        cur_v = cur.v;
+        nt = cur.nt;
+        q0w = cur.m0 + wave * kResident;
       }
-      const int t = s0; s0 = s1; s1 = s2; s2 = t;
+      qi = q0w + i;
+      ntw = nt;
+      if (CAUSAL) {
+        ntw = min(nt, (min(q0w + kResident, N) - 1) / kTile + 1);
+        if (q0w >= N) ntw = 0;
+      }
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+      m_run = -INFINITY;
+      l_run = 0.f;
+      auto wait_and_sync = [&]() __attribute__((always_inline)) {
+        if (in_flight == 2 * kIPW) wait_vm<2 * kIPW>();
+        else if (in_flight == kIPW) wait_vm<kIPW>();
+        else wait_vm<0>();
+        block_barrier();
+      };
+      auto compute = [&](int j, auto drain_tag) __attribute__((always_inline)) {
+        constexpr bool kDrain = decltype(drain_tag)::value != 0;
+        const char* Kl = k_ring + s0 * T::kBytes;
+        const char* Vl = v_ring + s2 * T::kBytes;
+        if (kFirst) {
+          accumulate(Vl, j - 1);
+          if (!kDrain) { scores(Kl, j); softmax(j); }
+        } else {
+          softmax(j - 1);
+          accumulate(Vl, j - 1);
+          if (!kDrain) scores(Kl, j);
+        }
+        if (!kDrain) { const int t = s0; s0 = s1; s1 = s2; s2 = t; }
+      };
+      // main part: both tiles to copy belong to this block
+      int j = 0;
+      for (; j + 2 < nt; ++j) {
+        wait_and_sync();
+        if (j == 0 && negate_q) {
+#pragma unroll
+          for (int kk = 0; kk < G::kKSteps; ++kk) qf[kk] = -qf[kk];
+        }
+        copy_tile(cur_k, ks.n, c_kgoff, k_ring + s2 * T::kBytes, j + 2);
+        copy_tile(cur_v, vs.n, c_vgoff, v_ring + s1 * T::kBytes, j + 1);
+        in_flight = 2 * kIPW;
+        compute(j, IntTag<0>{});
+      }
+      // tail: the last two tiles, during which the first tiles of the next block are copied
+      const int round_next = pb.next_round(round);
+      const int lin_next = round_next >= 0 ? pb.lin(round_next) : -1;
+      int pre_k = 0, pre_v = 0;  // tiles of the next block already issued
+      {
+        Block nxt = decode(lin_next >= 0 ? lin_next : lin_cur);
+        for (; j < nt; ++j) {
+          wait_and_sync();
+          if (j == 0 && negate_q) {
+#pragma unroll
+            for (int kk = 0; kk < G::kKSteps; ++kk) qf[kk] = -qf[kk];
+          }
+          in_flight = 0;
+          const int ek = j + 2, ev = j + 1;
+          if (ek < nt) {
+            copy_tile(cur_k, ks.n, c_kgoff, k_ring + s2 * T::kBytes, ek);
+            in_flight += kIPW;
+          } else if (lin_next >= 0 && ek - nt == pre_k && pre_k < min(2, nxt.nt)) {
+            copy_tile(nxt.k, ks.n, c_kgoff, k_ring + s2 * T::kBytes, pre_k);
+            ++pre_k;
+            in_flight += kIPW;
+          }
+          if (ev < nt) {
+            copy_tile(cur_v, vs.n, c_vgoff, v_ring + s1 * T::kBytes, ev);
+            in_flight += kIPW;
+          } else if (lin_next >= 0 && ev - nt == pre_v && pre_v < 1) {
+            copy_tile(nxt.v, vs.n, c_vgoff, v_ring + s1 * T::kBytes, 0);
+            ++pre_v;
+            in_flight += kIPW;
+          }
+          compute(j, IntTag<0>{});
+        }
+        // The last iteration has no tile of its own, only the second half of tile nt - 1.  Q was last used
+        // by scores(nt - 1), an iteration ago: the next block's rows are loaded over it.  This is a separate
+        // copy of the code so that, in the compiler's eyes, those loads never flow into a use of Q without the
+        // wait at the top of the next block between them.
+        wait_and_sync();
+        in_flight = 0;
+        if (lin_next >= 0) load_q(nxt);
+        compute(nt, IntTag<1>{});
+      }
+      // the block's output: O rows through this wave's staging tile, 64 features at a time
+      {
+        const Block cur = decode(lin_cur);
+        const float l_tot = l_run + other_half(l_run);
+        const float inv = 1.f / l_tot;
+#pragma unroll
+        for (int part = 0; part < D / 64; ++part)
+          store_resident<64>(O + cur.o_off + part * 64, rs, q0w, N, *reinterpret_cast<const f16v(*)[2]>(&o[2 * part]),
+                             inv, lane, stage);
+        if (hh == 0 && qi < N) LSE[cur.stat_off + qi] = (m_run * c + __builtin_amdgcn_logf(l_tot)) * kLn2;
+      }
+      if (lin_next < 0) break;
+      lin_cur = lin_next;
+      round = round_next;
+      {
+        // what a short previous block could not prefetch
+        const Block cur = decode(lin_cur);
+        if (pre_k < 1) copy_tile(cur.k, ks.n, c_kgoff, k_ring + s0 * T::kBytes, 0);
+        if (pre_k < 2 && cur.nt > 1) copy_tile(cur.k, ks.n, c_kgoff, k_ring + s1 * T::kBytes, 1);
+        if (pre_v < 1) copy_tile(cur.v, vs.n, c_vgoff, v_ring + s0 * T::kBytes, 0);
+      }
+      in_flight = 0;
     }
   };
   // Each group runs its own copy of the loop: no joins between the two
   // orders inside the loop, so no register shuffling at branch merges.
   if (first_group) run(IntTag<0>{});
   else run(IntTag<1>{});
-
-  const float l_tot = l_run + other_half(l_run);
-  const float inv = 1.f / l_tot;
-  static_assert(kFwdWaves * StageGeom<D>::kBytes <= 2 * kRing * T::kBytes, "the output staging tiles fit the rings");
-  block_barrier();  // every wave is done with the rings: they become the staging tiles
-  store_resident<D>(O + head_off, rs, q0w, N, o, inv, lane, smem + wave * StageGeom<D>::kBytes);
-  if (hh == 0 && qi < N) LSE[((long)b * H + h) * N + qi] = (m_run * c + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }
 
 // ---------------------------------------------------------------------------
@@ -1139,11 +1259,7 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
           half_t* dst = ds_lane + (long)(t >> 1) * np * 128 + (t & 1) * 2048;
 #pragma unroll
           for (int c16 = 0; c16 < 4; ++c16) {
-#if DS_NT_STORE
-            __builtin_nontemporal_store(y[c16], reinterpret_cast<h8*>(dst + c16 * 512));
-#else
-            *reinterpret_cast<h8*>(dst + c16 * 512) = y[c16];
-#endif
+            __builtin_nontemporal_store(y[c16], reinterpret_cast<h8*>(dst + c16 * 512));  // read once, later
           }
         }
       }
@@ -1176,17 +1292,21 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 // ---------------------------------------------------------------------------
 // Backward, dQ from spilled dS: dQ = scale * dS K, one GEMM, for callers whose
 // workspace holds the dS tiles fmha_bwd_dkdv_kernel<.., SPILL> wrote (layout there).
-// Block = 128 queries, 8 waves; wave w owns the 32 queries qb = w & 3 of the block
-// and half of the features (w >> 2), and computes per 64 keys
+// A block is 128 queries; of the 8 waves, wave w owns the 32 queries qb = w & 3 of the
+// block and half of the features (w >> 2), and computes per 64 keys
 //     dQ^T[d][q] += K^T[d][key] dS^T[key][q]
 // with both operands read transposed out of LDS (the K tile as everywhere else, the
-// dS tile as its 1 KiB pieces of [32 keys][16 queries]), so the order of the keys
-// inside a 16-key step is the same for both.
-// The kernel is bound by reading dS from HBM once, so what matters is the number of
-// bytes in flight: the 16 KiB dS tiles go through a 6-slot ring, five tiles ahead,
-// copied by waves 0-3 only; the K tiles (L2 hits) through a 3-slot ring, two ahead,
-// copied by waves 4-7 only.  A wave's copies complete in order, so a wave that issued
-// both would have to wait for young dS copies whenever it needs an older K tile.
+// dS tile as its 1 KiB pieces), so the order of the keys inside a 16-key step is the
+// same for both.
+// The kernel is bound by reading dS from HBM once, so what matters is that the stream
+// of tile copies never stops: the launch is persistent (PersistentBlocks) and the tiles
+// of a work group's blocks form ONE sequence that runs through the rings without regard
+// to block boundaries; an output block leaves through staging tiles of its own while
+// the copies of the next blocks' tiles are already in flight.  The 16 KiB dS tiles go
+// through a 5-slot ring, four tiles ahead, copied by waves 0-3 only; the K tiles (L2
+// hits) through a 3-slot ring, two ahead, copied by waves 4-7 only.  A wave's copies
+// complete in order, so a wave that issued both would have to wait for young dS copies
+// whenever it needs an older K tile.
 // The queries of a chunk sit in the order the dK/dV pass's registers held them (bits
 // 2 and 3 of the position inside 16 swapped); the epilogue puts the rows back in place.
 // (formula: reference kernel/fused_mha_kernel.cu:680-683.)
@@ -1194,25 +1314,22 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 constexpr int kDsWaves = 8;
 constexpr int kDsThreads = kDsWaves * 64;
 constexpr int kDsBlockQ = 128;
-#ifndef DQS_RING_S
-#define DQS_RING_S 6
-#define DQS_RING_K 3
-#define DQS_OCC 1
-#endif
-constexpr int kDsRingS = DQS_RING_S;   // dS tiles
-constexpr int kDsRingK = DQS_RING_K;   // K tiles
+constexpr int kDsRingS = 5;   // dS tiles
+constexpr int kDsRingK = 3;   // K tiles
 constexpr int kDsTileBytes = kTile * kDsBlockQ * 2;
+constexpr int kDsStageD = 32;          // features staged at a time in the epilogue
 
 template <int D, bool CAUSAL>
-__global__ void __launch_bounds__(kDsThreads, DQS_OCC)
+__global__ void __launch_bounds__(kDsThreads, 1)
 fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t* __restrict__ dS, int np,
-                         half_t* __restrict__ dQ, int H, int N, int nqb, float scale) {
+                         half_t* __restrict__ dQ, int H, int N, int nqb, int total, float scale) {
   using T = SwzTile<D>;             // K tile: 64 keys x D features
   constexpr int kCopyWaves = kDsWaves / 2;
   constexpr int kKIPW = T::kInstrs / kCopyWaves;           // K copies per K-copying wave and tile
   constexpr int kSIPW = (kDsTileBytes / 1024) / kCopyWaves;  // dS copies per dS-copying wave and tile
   constexpr int kDBW = D / 64;      // 32-feature blocks per wave
-  __shared__ __attribute__((aligned(1024))) char smem[kDsRingS * kDsTileBytes + kDsRingK * T::kBytes];
+  constexpr int kStageBytes = StageGeom<kDsStageD>::kBytes;
+  __shared__ __attribute__((aligned(1024))) char smem[kDsRingS * kDsTileBytes + kDsRingK * T::kBytes + kDsWaves * kStageBytes];
   char* const s_ring = smem;
   char* const k_ring = smem + kDsRingS * kDsTileBytes;
 
@@ -1222,19 +1339,46 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
   const bool copies_k = wave >= kCopyWaves;
   const int cw = wave & (kCopyWaves - 1);
   const int i = lane & 31;
-  int bh, mb;
-  slice_and_block(nqb, bh, mb);
-  const int mblk = CAUSAL ? nqb - 1 - mb : mb;  // heavy blocks first
-  const int b = bh / H, h = bh - b * H;
+  char* const stage = smem + kDsRingS * kDsTileBytes + kDsRingK * T::kBytes + wave * kStageBytes;
   const int rs = H * D;  // dQ is dense
-  const long head_off = ((long)b * N * H + h) * D;
-  const half_t* Kb = K + b * ks.b + (long)h * ks.h;
-  const half_t* Sb = dS + (((long)bh * nqb + mblk) * np) * kDsBlockQ;  // this block's np / 64 tiles of 16 KiB
-
   const int nt_all = (N + kTile - 1) / kTile;
-  const int nt = CAUSAL ? min(nt_all, 2 * mblk + 2) : nt_all;  // tiles the block streams
-  const int qt = 2 * mblk + (qb >> 1);                         // this wave's query tile
-  const int jend = qt >= nt_all ? 0 : (CAUSAL ? min(nt, qt + 1) : nt);  // tiles this wave takes part in
+  const int slices = total / nqb;
+  const PersistentBlocks pb{total};
+
+  // A position in the work group's sequence of tiles: block (round, number), tile j of its nt.
+  struct Cursor {
+    int round, lin, j, nt, mblk;
+    const half_t* base;  // the block's dS panel (consumer and dS copies) or the slice's K rows (K copies)
+    long out_off;        // consumer: element offset of the slice in dQ
+  };
+  auto open = [&](int round, bool for_k) __attribute__((always_inline)) {
+    Cursor c;
+    c.round = round;
+    c.lin = round >= 0 ? pb.lin(round) : 0;
+    int bh, mb;
+    fmha_slice_and_block(c.lin, slices, nqb, bh, mb);
+    c.mblk = CAUSAL ? nqb - 1 - mb : mb;  // heavy blocks first
+    const int b = bh / H, h = bh - b * H;
+    c.j = 0;
+    c.nt = CAUSAL ? min(nt_all, 2 * c.mblk + 2) : nt_all;
+    c.base = for_k ? K + b * ks.b + (long)h * ks.h : dS + (((long)bh * nqb + c.mblk) * np) * kDsBlockQ;
+    c.out_off = ((long)b * N * H + h) * D;
+    return c;
+  };
+  auto advance = [&](Cursor& c, bool for_k) __attribute__((always_inline)) {  // to the next tile of the sequence
+    if (++c.j == c.nt) {
+      const int r = pb.next_round(c.round);
+      if (r >= 0) c = open(r, for_k);
+      else c.round = -1;  // past the end
+    }
+  };
+  int n_tiles = 0;  // tiles in this work group's sequence
+  for (int r = 0; r >= 0; r = pb.next_round(r)) {
+    int bh, mb;
+    fmha_slice_and_block(pb.lin(r), slices, nqb, bh, mb);
+    const int mblk = CAUSAL ? nqb - 1 - mb : mb;
+    n_tiles += CAUSAL ? min(nt_all, 2 * mblk + 2) : nt_all;
+  }
 
   // K copies: this wave's share of a tile (as in the other kernels).  dS copies: piece p = cw * kSIPW + u of
   // the tile, 1 KiB, lane l fetching 16 bytes.  In memory a piece is [2 halves][32 keys] x 16 bytes; in LDS it
@@ -1255,15 +1399,15 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
     const int at = (piece & 1) ? (lane - 8) & 63 : lane;  // position (key, half) = (at >> 1, at & 1) of the piece in LDS
     c_sgoff[u] = piece * 1024 + ((at & 1) * 32 + (at >> 1)) * 16;
   }
-  auto copy_s = [&](int j, int slot) __attribute__((always_inline)) {
-    const half_t* sp = Sb + (long)j * (kDsTileBytes / 2);  // wave-uniform
+  auto copy_s = [&](const Cursor& c, int slot) __attribute__((always_inline)) {
+    const half_t* sp = c.base + (long)c.j * (kDsTileBytes / 2);  // wave-uniform
     char* dst = s_ring + slot * kDsTileBytes + cw * kSIPW * 1024;
 #pragma unroll
     for (int u = 0; u < kSIPW; ++u) copy16_stream(sp, c_sgoff[u], dst + u * 1024);
   };
-  auto copy_k = [&](int j, int slot) __attribute__((always_inline)) {
-    const int row0 = j * kTile;
-    const half_t* kp = Kb + (long)row0 * ks.n;  // wave-uniform
+  auto copy_k = [&](const Cursor& c, int slot) __attribute__((always_inline)) {
+    const int row0 = c.j * kTile;
+    const half_t* kp = c.base + (long)row0 * ks.n;  // wave-uniform
     char* dst = k_ring + slot * T::kBytes;
     if (row0 + kTile <= N) {
 #pragma unroll
@@ -1276,12 +1420,6 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
       }
     }
   };
-  constexpr int kAheadS = kDsRingS - 1, kAheadK = kDsRingK - 1;
-  if (copies_k) {
-    for (int j = 0; j < kAheadK && j < nt; ++j) copy_k(j, j);
-  } else {
-    for (int j = 0; j < kAheadS && j < nt; ++j) copy_s(j, j);
-  }
 
   // LDS offsets of this lane's transposing reads.  K tile: as in the other kernels.  dS tile: key step kc,
   // read e: key row (kc & 1) * 16 + 8 * e + 4 * hhk + (L >> 2) of the piece [(kc >> 1)][query tile][chunk
@@ -1312,21 +1450,37 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
   for (int db = 0; db < kDBW; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
+  // column i of the accumulator is the query at position i of the wave's 32: bits 2 and 3 swapped
+  const int my_row = (i & 0x13) | ((i & 8) >> 1) | ((i & 4) << 1);
 
-  int slot_s = 0, slot_k = 0;                        // ring slots of tile j
+  constexpr int kAheadS = kDsRingS - 1, kAheadK = kDsRingK - 1;
+  // the copying waves run ahead of the sequence: kAhead tiles are issued before the first is used
+  Cursor ahead = open(0, copies_k);
+  {
+    const int n_first = min(copies_k ? kAheadK : kAheadS, n_tiles);
+    for (int t = 0; t < n_first; ++t) {
+      if (copies_k) copy_k(ahead, t);
+      else copy_s(ahead, t);
+      advance(ahead, copies_k);
+    }
+  }
+  Cursor cur = open(0, false);
+  int slot_s = 0, slot_k = 0;                                    // ring slots of tile t
   int next_s = kAheadS % kDsRingS, next_k = kAheadK % kDsRingK;  // ring slots of the tiles to copy next
-  for (int j = 0; j < nt; ++j) {
-    // tile j must have landed; the copies of the tiles after it (at most kAhead - 1 of them) may be in flight
-    const int later = nt - 1 - j;
+  for (int t = 0; t < n_tiles; ++t) {
+    // tile t must have landed; the copies of the tiles after it (at most kAhead - 1 of them) may be in flight
+    const int later = n_tiles - 1 - t;
     if (copies_k) wait_vm_tiles<kKIPW, kAheadK - 1>(later);
     else wait_vm_tiles<kSIPW, kAheadS - 1>(later);
-    block_barrier();  // tile j is visible to all; everybody is done with tile j - 1, whose slots are reused now
-    if (copies_k) {
-      if (j + kAheadK < nt) copy_k(j + kAheadK, next_k);
-    } else {
-      if (j + kAheadS < nt) copy_s(j + kAheadS, next_s);
+    block_barrier();  // tile t is visible to all; everybody is done with tile t - 1, whose slots are reused now
+    if (ahead.round >= 0) {
+      if (copies_k) copy_k(ahead, next_k);
+      else copy_s(ahead, next_s);
+      advance(ahead, copies_k);
     }
-    if (j < jend) {
+    const int qt = 2 * cur.mblk + (qb >> 1);                                      // this wave's query tile
+    const int jend = qt >= nt_all ? 0 : (CAUSAL ? min(cur.nt, qt + 1) : cur.nt);  // tiles this wave takes part in
+    if (cur.j < jend) {
       const char* Kl = k_ring + slot_k * T::kBytes;
       const char* Sl = s_ring + slot_s * kDsTileBytes;
 #pragma unroll
@@ -1337,17 +1491,23 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
           acc[db] = mfma(swz_cols<D>(Kl, c16, dh * kDBW + db, c_off), bfrag, acc[db]);
       }
     }
+    if (cur.j == cur.nt - 1) {  // the block's last tile: its rows leave through this wave's staging tile
+      half_t* out = dQ + cur.out_off + dh * (D / 2);
+      const int row0 = cur.mblk * kDsBlockQ + qb * kResident;
+#pragma unroll
+      for (int part = 0; part < kDBW; ++part) {
+        store_resident<kDsStageD>(out + part * kDsStageD, rs, row0, N, *reinterpret_cast<const f16v(*)[1]>(&acc[part]),
+                                  scale, lane, stage, my_row);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[part][r] = 0.f;
+      }
+    }
+    advance(cur, false);
     slot_s = slot_s + 1 == kDsRingS ? 0 : slot_s + 1;
     slot_k = slot_k + 1 == kDsRingK ? 0 : slot_k + 1;
     next_s = next_s + 1 == kDsRingS ? 0 : next_s + 1;
     next_k = next_k + 1 == kDsRingK ? 0 : next_k + 1;
   }
-  static_assert(kDsWaves * StageGeom<D / 2>::kBytes <= kDsRingS * kDsTileBytes, "the output staging tiles fit the ring");
-  block_barrier();  // every wave is done with the rings: they become the staging tiles
-  // column i of the accumulator is the query at position i of the wave's 32: bits 2 and 3 swapped
-  const int my_row = (i & 0x13) | ((i & 8) >> 1) | ((i & 4) << 1);
-  store_resident<D / 2>(dQ + head_off + dh * (D / 2), rs, mblk * kDsBlockQ + qb * kResident, N, acc, scale, lane,
-                        smem + wave * StageGeom<D / 2>::kBytes, my_row);
 }
 
 // ---------------------------------------------------------------------------
@@ -1379,6 +1539,26 @@ hipError_t launch(void (*kernel)(Params...), unsigned grid, unsigned block, hipS
   return hipLaunchKernel((const void*)kernel, dim3(grid), dim3(block), ptrs, 0, stream);
 }
 
+// Work groups of a persistent launch over `total` blocks: one per CU of the current device,
+// rounded down to a multiple of 8 (the XCDs take work-group ids round-robin), or one per block
+// when there are no more blocks than that.
+unsigned persistent_grid(int total) {
+  static std::mutex mu;
+  static int cus[64] = {};
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+    std::lock_guard<std::mutex> lock(mu);
+    if (!cus[dev]) {
+      int v = 0;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus[dev] = v;
+    }
+    n = cus[dev];
+  }
+  if (n < 8) n = 256;  // the query failed: MI355X has 256
+  n &= ~7;
+  return (unsigned)(total <= n ? total : n);
+}
+
 bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
 
 // Strides from the C structure, or the dense layout when the caller gave none.
@@ -1400,12 +1580,13 @@ template <int D, bool CAUSAL>
 int launch_forward(const void* q, const void* k, const void* v, Strides qs, Strides ks, Strides vs, void* o, void* lse,
                    int batch, int head, int n, float scale, hipStream_t stream) {
   const int nmb = (n + kFwdBlockQ - 1) / kFwdBlockQ;
-  const unsigned grid = (unsigned)nmb * batch * head;
+  const int total = nmb * batch * head;
+  const unsigned grid = persistent_grid(total);
   // scale == 0 would turn the masked scores (-inf) into NaN when multiplied; a
   // tiny positive factor gives the same uniform softmax and keeps -inf * c = -inf.
   const float c = fmaxf(fabsf(scale) * kLog2e, 1e-30f);
   const hipError_t rc = launch(fmha_fwd_kernel<D, CAUSAL>, grid, kFwdThreads, stream, (const half_t*)q,
-                               (const half_t*)k, (const half_t*)v, qs, ks, vs, (half_t*)o, (float*)lse, head, n, nmb, c,
+                               (const half_t*)k, (const half_t*)v, qs, ks, vs, (half_t*)o, (float*)lse, head, n, nmb, total, c,
                                scale < 0.f ? 1 : 0);
   return rc == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
 }
@@ -1459,9 +1640,9 @@ int launch_backward(int passes, bool spill, const void* q, const void* k, const 
   const float c = scale * kLog2e;
   auto dq_pass = [&]() {
     if (spill) {
-      const int nqb = np / kDsBlockQ;
-      return launch(fmha_bwd_dq_spill_kernel<D, CAUSAL>, (unsigned)nqb * batch * head, kDsThreads, stream,
-                    (const half_t*)k, ks, (const half_t*)ds, np, (half_t*)dq, head, n, nqb, scale);
+      const int nqb = np / kDsBlockQ, total = nqb * batch * head;
+      return launch(fmha_bwd_dq_spill_kernel<D, CAUSAL>, persistent_grid(total), kDsThreads, stream,
+                    (const half_t*)k, ks, (const half_t*)ds, np, (half_t*)dq, head, n, nqb, total, scale);
     }
     const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;
     auto kernel = dq_makes_stats ? fmha_bwd_dq_kernel<D, CAUSAL, true> : fmha_bwd_dq_kernel<D, CAUSAL, false>;
