@@ -26,6 +26,7 @@ PEAK_TFLOPS = 2516.6  # MI355X dense fp16 MFMA, vendor figure (256 CUs x 4 SIMDs
 NOMINAL_MHZ = 2400
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E, vendor figure
 SUSTAINED_LAUNCHES = 300
+SETTLE_MS = 100.0  # untimed load before the warm-up steps (power management ramp)
 
 CONFIGS = [  # name, B, H, N, D, causal
     ("plumbing_b1_h4_n128_d64", 1, 4, 128, 64, False),
@@ -63,6 +64,8 @@ def load_c_abi():
     lib.fused_mha_forward.argtypes = [vp] * 5 + [i] * 5 + [f, i, vp]
     lib.fused_mha_backward_workspace_bytes.argtypes = [i] * 4
     lib.fused_mha_backward_workspace_bytes.restype = sz
+    lib.fused_mha_backward_min_workspace_bytes.argtypes = [i] * 4
+    lib.fused_mha_backward_min_workspace_bytes.restype = sz
     lib.fused_mha_backward_delta.argtypes = [vp, vp, vp, vp, sz] + [i] * 4 + [vp]
     lib.fused_mha_backward_dq.argtypes = [vp] * 6 + [sz, vp] + [i] * 4 + [f, i, vp]
     lib.fused_mha_backward_dkdv.argtypes = [vp] * 6 + [sz, vp, vp] + [i] * 4 + [f, i, vp]
@@ -196,7 +199,7 @@ def occupancy_sweep(path):
     scale = 1.0 / math.sqrt(D)
     with open(path, "w") as fh:
         fh.write("# B1 N4096 D128 non-causal; medians of 100 launches, microseconds; 256 CUs; work groups per kernel:\n")
-        fh.write("# forward heads*16 (256 queries each), dQ and dK/dV heads*32 (128 rows each)\n")
+        fh.write("# forward heads*16 blocks (256 queries each), dQ and dK/dV heads*32 (128 rows each); forward and dQ launches are persistent\n")
         fh.write("# heads fwd_groups fwd_us fwd_us_per_round dq_us dkdv_us\n")
         for H in (2, 4, 8, 16, 32, 64):
             q, k, v, do = make_device_inputs(B, H, N, D)
@@ -210,14 +213,14 @@ def occupancy_sweep(path):
             calls = [
                 lambda: lib.fused_mha_forward(p(q), p(k), p(v), p(out), p(lse), B, H, N, N, D, scale, 0, s),
                 lambda: lib.fused_mha_backward_delta(p(out), p(do), p(lse), p(ws), nbytes, B, H, N, D, s),
-                lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dq), B, H, N, D, scale, 0, s),
                 lambda: lib.fused_mha_backward_dkdv(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dk), p(dv),
                                                     B, H, N, D, scale, 0, s),
+                lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dq), B, H, N, D, scale, 0, s),
             ]
-            for fn in calls:
+            for fn in calls:  # in dependency order: the dQ pass reads the dS tiles the dK/dV pass wrote
                 if fn() != 0:
                     sys.exit("bench.py: a kernel of the occupancy sweep failed")
-            us = [sustained_ms(fn, 100, 20)[0] * 1e3 for fn in (calls[0], calls[2], calls[3])]
+            us = [sustained_ms(fn, 100, 20)[0] * 1e3 for fn in (calls[0], calls[3], calls[2])]
             groups = H * N // 256
             rounds = max(1, -(-groups // 256))
             fh.write("%d %d %.1f %.1f %.1f %.1f\n" % (H, groups, us[0], us[0] / rounds, us[1], us[2]))
@@ -258,7 +261,10 @@ def bench_config(B, H, N, D, causal, steps, warmup):
 
 
 def kernel_times(B, H, N, D, causal, steps, warmup):
-    """Average duration of each kernel, timed one by one through the C ABI."""
+    """Average duration of each kernel of the path flash_attn_func takes, timed one by one through the C ABI with
+    device events on the launch stream: forward; delta; the dK/dV pass that also writes the dS tiles; the dQ pass
+    that reads them.  `fmha_bwd_dq_kernel` (the dQ pass of the minimum-workspace path, which recomputes S and dP) is
+    timed beside them for comparison."""
     import torch
 
     lib = load_c_abi()
@@ -267,19 +273,24 @@ def kernel_times(B, H, N, D, causal, steps, warmup):
     out = torch.empty_like(q)
     lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
     nbytes = lib.fused_mha_backward_workspace_bytes(B, H, N, D)
+    small = lib.fused_mha_backward_min_workspace_bytes(B, H, N, D)
     ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)
     s = torch.cuda.current_stream().cuda_stream
     p = lambda t: t.data_ptr()
     c = int(causal)
+    spill = nbytes > small
     calls = {
         "fmha_fwd_kernel": lambda: lib.fused_mha_forward(p(q), p(k), p(v), p(out), p(lse), B, H, N, N, D, scale, c, s),
         "fmha_bwd_delta_kernel": lambda: lib.fused_mha_backward_delta(p(out), p(do), p(lse), p(ws), nbytes, B, H, N, D, s),
-        "fmha_bwd_dq_kernel": lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dq),
-                                                                 B, H, N, D, scale, c, s),
         "fmha_bwd_dkdv_kernel": lambda: lib.fused_mha_backward_dkdv(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes,
                                                                      p(dk), p(dv), B, H, N, D, scale, c, s),
+        ("fmha_bwd_dq_spill_kernel" if spill else "fmha_bwd_dq_kernel"):
+            lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), nbytes, p(dq), B, H, N, D, scale, c, s),
     }
+    if spill:
+        calls["fmha_bwd_dq_kernel"] = lambda: lib.fused_mha_backward_dq(p(q), p(k), p(v), p(do), p(lse), p(ws), small,
+                                                                         p(dq), B, H, N, D, scale, c, s)
     for name, fn in calls.items():  # each pass once, in dependency order, and every return code checked
         rc = fn()
         if rc != 0:
@@ -344,9 +355,6 @@ def main():
                          "(launch index, milliseconds since the first launch, duration in milliseconds)")
     ap.add_argument("--launch-trace-count", type=int, default=6000,
                     help="launches in the --launch-trace run (default 6000, about two seconds)")
-    ap.add_argument("--microbench", metavar="FILE",
-                    help="first run the stand-alone programs of flash-attention-v100_amd/microbench/bin (instruction "
-                         "issue and MFMA rates, atomic-add throughput) and write what they print to FILE")
     ap.add_argument("--occupancy-sweep", metavar="FILE",
                     help="write kernel durations of B1 N4096 D128 for 2 .. 64 heads (32 .. 1024 forward work groups) to FILE")
     ap.add_argument("--no-clock-sample", action="store_true", help="do not read the shader clock under load (rocm-smi)")
@@ -355,18 +363,6 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus)
-
-    if args.microbench:  # child processes: started before this process touches the GPU
-        import subprocess
-
-        with open(args.microbench, "w") as fh:
-            for prog in ("issue_rate", "atomic_add"):
-                exe = os.path.join(ROOT, "flash-attention-v100_amd", "microbench", "bin", prog)
-                if not os.path.exists(exe):
-                    sys.exit("bench.py: %s is not built (python flash-attention-v100_amd/setup.py build_microbench)" % exe)
-                fh.write("== %s\n" % prog)
-                fh.flush()
-                subprocess.run([exe], stdout=fh, stderr=subprocess.STDOUT, timeout=120, check=True)
 
     # (not under a profiler: its preloaded library has initialised the GPU before this program started)
     profiled = "rocprof" in os.environ.get("LD_PRELOAD", "") or any(key.startswith("ROCPROF") for key in os.environ)
@@ -398,6 +394,14 @@ def main():
         out.backward(do)
         q.grad = k.grad = v.grad = None
 
+    # After an idle period the first 20-30 ms of load run slower while the power management ramps up
+    # (profiles/headline_forward_launch_index_vs_duration.md), whatever --warmup says: SETTLE_MS of untimed steps
+    # come first, then the --warmup steps, then the timed ones.
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < SETTLE_MS:
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -451,15 +455,20 @@ def main():
     kt = kernel_times(B, H, N, D, causal, args.steps, args.warmup)
     # algorithmic FLOPs per launch: the GEMMs of the 5-GEMM backward / 2-GEMM forward
     # count that each kernel produces (recomputed S and dP in the dQ pass are not counted)
-    alg = {"fmha_fwd_kernel": ff, "fmha_bwd_dkdv_kernel": 2.0 * ff, "fmha_bwd_dq_kernel": 0.5 * ff}
-    dominant = max(alg, key=lambda n: kt[n])
+    alg = {"fmha_fwd_kernel": ff, "fmha_bwd_dkdv_kernel": 2.0 * ff, "fmha_bwd_dq_spill_kernel": 0.5 * ff,
+           "fmha_bwd_dq_kernel": 0.5 * ff}
+    on_path = [n for n in alg if n in kt and not (n == "fmha_bwd_dq_kernel" and "fmha_bwd_dq_spill_kernel" in kt)]
+    dominant = max(on_path, key=lambda n: kt[n])
     achieved = alg[dominant] / kt[dominant] / 1e9
-    traffic = None
+    traffic = traffic_commit = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath) and args.config_index == HEADLINE:  # the counters were taken on the headline workload
-        traffic = json.load(open(tpath)).get(dominant)
+        tj = json.load(open(tpath))
+        traffic = tj.get(dominant)
+        traffic_commit = tj.get("_commit")
     roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_TFLOPS, "traffic": traffic,
+                "traffic_measured_at_commit": traffic_commit,
                 # the same against the peak at the shader clock measured under the fwd+bwd load (informative)
                 "frac_at_step_sclk": achieved / clock["peak_at_step_sclk_tflops"] if clock["peak_at_step_sclk_tflops"] else None,
                 "kernel_ms": kt, "peak_check_tflops": peak_check}
@@ -476,6 +485,7 @@ def main():
         "metric": "fwd+bwd TFLOP/s, B%d H%d N%d D%d %s fp16 (fwd alone in 'fwd')" % (
             B, H, N, D, "causal" if causal else "non-causal"),
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "settle_ms_before_warmup": SETTLE_MS,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": name, "batch": B, "heads": H, "seq_len": N, "head_dim": D, "causal": causal},

@@ -47,4 +47,22 @@ FMHA_HOST_DEVICE void fmha_slice_and_block(int lin, int slices, int blocks_per_s
     blk = idx - s * blocks_per_slice;
   }
 }
+
+// Persistent launches: G work groups (one per CU) share the `total` blocks numbered as above.
+// Work group w takes, in round r, block r * G + w for even r and r * G + (w mirrored inside its
+// XCD, i.e. among the work groups congruent to w modulo 8) for odd r.  Both keep the block number
+// congruent to w modulo 8, so the block stays on w's XCD, and the alternation pairs the heavy
+// blocks of one round with the light blocks of the next (blocks are numbered heaviest first).
+// G must be a multiple of 8 unless the launch has a single round (total <= G).
+// fmha_persistent_block: the block of work group w in round r; >= total means none.
+// fmha_persistent_next_round: the next round after r in which w has a block, or -1.
+FMHA_HOST_DEVICE int fmha_persistent_block(int r, int w, int G) {
+  const int p = (r & 1) ? (((G >> 3) - 1 - (w >> 3)) << 3) + (w & 7) : w;
+  return r * G + p;
+}
+FMHA_HOST_DEVICE int fmha_persistent_next_round(int r, int w, int G, int total) {
+  for (++r; (long)r * G < total; ++r)
+    if (fmha_persistent_block(r, w, G) < total) return r;
+  return -1;
+}
 #endif  // FMHA_BLOCK_MAP_H_

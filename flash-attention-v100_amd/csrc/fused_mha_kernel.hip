@@ -141,23 +141,14 @@ __device__ __forceinline__ void slice_and_block(int blocks_per_slice, int& slice
   fmha_slice_and_block(blockIdx.x, gridDim.x / blocks_per_slice, blocks_per_slice, slice, blk);
 }
 
-// Blocks of a persistent work group.  The launch's blocks are numbered as by
-// fmha_slice_and_block (heaviest first inside every XCD's groups of slices); work group w of G
-// takes, in round r, block r * G + w for even r and r * G + (w mirrored inside its XCD) for odd r.
-// Both keep the block number congruent to w modulo 8, i.e. on w's XCD, and the alternation pairs
-// the heavy blocks of one round with the light blocks of the next.  G is a multiple of 8 unless
-// the launch has a single round.
+// Blocks of a persistent work group (schedule: block_map.h).
 struct PersistentBlocks {
   int total;
   __device__ __forceinline__ int lin(int r) const {  // >= total: this group has no block in round r
-    const int G = gridDim.x, w = blockIdx.x;
-    const int p = (r & 1) ? (((G >> 3) - 1 - (w >> 3)) << 3) + (w & 7) : w;
-    return r * G + p;
+    return fmha_persistent_block(r, blockIdx.x, gridDim.x);
   }
   __device__ __forceinline__ int next_round(int r) const {  // the next round with a block for this group, or -1
-    for (++r; (long)r * gridDim.x < total; ++r)
-      if (lin(r) < total) return r;
-    return -1;
+    return fmha_persistent_next_round(r, blockIdx.x, gridDim.x, total);
   }
 };
 
@@ -1513,15 +1504,22 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
 // ---------------------------------------------------------------------------
 // Host side: validation and launches.
 // ---------------------------------------------------------------------------
-// Limits of the 32-bit arithmetic in the kernels: a (batch, head) row of lse /
-// delta is addressed with 32-bit byte offsets (n < 2^29), and the 1-D grid of
-// the finest pass (128-row blocks) must fit a launch (below 2^31 work groups).
+// Limits of the 32-bit arithmetic in the kernels and of what a launch can take:
+//   - a (batch, head) row of lse / delta is addressed with 32-bit byte offsets (n < 2^29);
+//   - the dense row stride head * d and the per-lane byte offsets built from it are 32-bit
+//     (head * d < 2^24, the bound the strided entry points put on the sequence stride);
+//   - a launch holds fewer than 2^32 threads: the finest non-persistent grids are the 128-row
+//     blocks of the backward at 512 threads each (fewer than 2^23 blocks) and the delta pass
+//     at one thread per 8 features of a row (batch * head * n * d / 8 < 2^32).
+// Checked up front, so that nothing is enqueued for a problem a later pass would refuse.
 int check_shape(int batch, int head, int m, int n, int d) {
   if (batch <= 0 || head <= 0 || n <= 0 || m != n) return FUSED_MHA_ERR_BAD_SHAPE;
   if (d != 64 && d != 128) return FUSED_MHA_ERR_BAD_HEAD_DIM;
   if (n >= (1 << 29)) return FUSED_MHA_ERR_TOO_LARGE;
+  if ((long)head * d >= (1L << 24)) return FUSED_MHA_ERR_TOO_LARGE;
   const long blocks = (long)((n + 127) / 128) * batch * head;
-  if (blocks >= (1L << 31)) return FUSED_MHA_ERR_TOO_LARGE;
+  if (blocks >= (1L << 23)) return FUSED_MHA_ERR_TOO_LARGE;
+  if ((long)batch * head * n * (d / 8) >= (1L << 32)) return FUSED_MHA_ERR_TOO_LARGE;
   return FUSED_MHA_OK;
 }
 
@@ -1819,7 +1817,9 @@ const char* fused_mha_error_string(int code) {
     case FUSED_MHA_ERR_MISALIGNED: return "a pointer is not 16-byte aligned";
     case FUSED_MHA_ERR_LAUNCH: return "the HIP runtime refused a kernel launch";
     case FUSED_MHA_ERR_BAD_SCALE: return "scale must be finite";
-    case FUSED_MHA_ERR_TOO_LARGE: return "problem too large: need n < 2^29 and ceil(n/128) * batch * head < 2^31";
+    case FUSED_MHA_ERR_TOO_LARGE:
+      return "problem too large: need n < 2^29, head * d < 2^24, ceil(n/128) * batch * head < 2^23 and "
+             "batch * head * n * d / 8 < 2^32";
     case FUSED_MHA_ERR_BAD_STRIDE:
       return "strides must be non-negative multiples of 8 elements, sequence stride below 2^24, head stride below 2^31";
     case FUSED_MHA_ERR_SCRATCH_LIMIT:

@@ -19,10 +19,6 @@ builds them in-tree, next to this file.  An install or wheel build reuses in-tre
 artefacts that are newer than every source and compiles otherwise
 (FLASH_ATTN_FORCE_BUILD=1 always compiles).
 The functions build_kernels() / build_extension() can also be imported.
-
-    python setup.py build_microbench
-compiles the two stand-alone measurement programs of microbench/ (instruction issue and MFMA
-rates; fp32 atomic-add throughput) into microbench/bin/; `bench.py --microbench FILE` runs them.
 """
 import os
 import shutil
@@ -88,23 +84,6 @@ def build_extension(out=EXT_LIB):
     return out
 
 
-MICROBENCH = os.path.join(HERE, "microbench")
-
-
-def build_microbench():
-    """Stand-alone HIP programs (no PyTorch): microbench/bin/issue_rate, microbench/bin/atomic_add."""
-    out_dir = os.path.join(MICROBENCH, "bin")
-    os.makedirs(out_dir, exist_ok=True)
-    hipcc = os.path.join(ROCM_HOME, "bin", "hipcc")
-    common = ["--offload-arch=gfx950", "-O2", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-              "-Wno-unused-command-line-argument"]
-    outs = []
-    for name, extra in (("issue_rate", []), ("atomic_add", ["-munsafe-fp-atomics"])):
-        outs.append(os.path.join(out_dir, name))
-        _run([hipcc, *common, *extra, "-o", outs[-1], os.path.join(MICROBENCH, name + ".hip")])
-    return outs
-
-
 def build_all():
     build_kernels()
     build_extension()
@@ -116,9 +95,6 @@ def _fresh(artefact, sources):
 
 
 if __name__ == "__main__":
-    if sys.argv[1:] == ["build_microbench"]:
-        build_microbench()
-        sys.exit(0)
     from setuptools import Extension, setup
     from setuptools.command.build_ext import build_ext as _build_ext
 

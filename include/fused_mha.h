@@ -22,6 +22,8 @@
  *   - stream is a hipStream_t passed as void*; NULL is the default stream.
  *     All work is enqueued asynchronously; nothing synchronises.
  *   - All pointers are borrowed device pointers and must be 16-byte aligned.
+ *   - Size limits (FUSED_MHA_ERR_TOO_LARGE otherwise): n < 2^29, head * d < 2^24,
+ *     ceil(n / 128) * batch * head < 2^23 and batch * head * n * d / 8 < 2^32.
  *   - Return value: FUSED_MHA_OK (0) or a negative FUSED_MHA_ERR_* code.
  *     Arguments are validated before anything is launched; only
  *     FUSED_MHA_ERR_LAUNCH can come back after part of the work (an earlier
@@ -43,7 +45,7 @@ extern "C" {
 #define FUSED_MHA_ERR_MISALIGNED (-4)     /* a pointer is not 16-byte aligned      */
 #define FUSED_MHA_ERR_LAUNCH (-5)         /* the HIP runtime refused the launch    */
 #define FUSED_MHA_ERR_BAD_SCALE (-6)      /* scale is NaN or infinite              */
-#define FUSED_MHA_ERR_TOO_LARGE (-7)      /* n >= 2^29 or more than 2^31-1 blocks  */
+#define FUSED_MHA_ERR_TOO_LARGE (-7)      /* beyond the limits listed below        */
 #define FUSED_MHA_ERR_BAD_STRIDE (-8)     /* see fused_mha_strides                 */
 #define FUSED_MHA_ERR_SCRATCH_LIMIT (-9)  /* see fused_mha_backward_noalloc        */
 #define FUSED_MHA_ERR_RUNTIME (-10)       /* a HIP runtime query failed            */
@@ -152,8 +154,10 @@ int fused_mha_backward_strided(const void *query_ptr, const fused_mha_strides *q
  * callers that cannot allocate device memory: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  It calls no hipMalloc,
  * hipFree or allocating library routine; the first call on a device looks up
- * the array's device address, every later call only launches the kernels of
- * fused_mha_backward.  Results are bit-identical to fused_mha_backward.
+ * the array's device address (which may make the runtime load the code
+ * object: make that one call outside graph capture), every later call only
+ * launches the kernels fused_mha_backward launches for a workspace of
+ * fused_mha_backward_min_workspace_bytes, with bit-identical results.
  *   - batch*head*n above FUSED_MHA_NOALLOC_MAX_ROWS: FUSED_MHA_ERR_SCRATCH_LIMIT.
  *   - The device that owns the tensors must be the current device.
  *   - All calls on one GPU share that GPU's array: calls that overlap in time

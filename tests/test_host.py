@@ -70,10 +70,17 @@ def test_forward_validation_codes(lib):
     assert f(p, p, p, p, p, 1, 1, 32, 32, 64, float("nan"), 0, None) == abi.ERR_BAD_SCALE
     assert f(p, p, p, p, p, 1, 1, 32, 32, 64, float("inf"), 0, None) == abi.ERR_BAD_SCALE
     assert f(p + 2, p, p, p, p, 1, 1, 32, 32, 64, 1.0, 0, None) == abi.ERR_MISALIGNED
-    # the limits of the kernels' 32-bit arithmetic: n < 2^29, ceil(n/128)*batch*head < 2^31
+    # the limits of the kernels' 32-bit arithmetic and of a launch: n < 2^29, head*d < 2^24,
+    # ceil(n/128)*batch*head < 2^23, batch*head*n*d/8 < 2^32
     assert f(p, p, p, p, p, 1, 1, 1 << 29, 1 << 29, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
     assert f(p, p, p, p, p, 1 << 12, 1 << 12, 1 << 14, 1 << 14, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
     assert f(p, p, p, p, p, 2048, 2048, 1 << 16, 1 << 16, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE
+    assert f(p, p, p, p, p, 1, 1 << 17, 128, 128, 128, 1.0, 0, None) == abi.ERR_TOO_LARGE    # head*d = 2^24
+    assert f(p, p, p, p, p, 1, 1 << 18, 128, 128, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE     # head*d = 2^24
+    assert f(p, p, p, p, p, 1 << 11, 1 << 12, 128, 128, 64, 1.0, 0, None) == abi.ERR_TOO_LARGE  # 2^23 blocks of 128 rows
+    assert f(p, p, p, p, p, 1 << 9, 1 << 12, 130, 130, 128, 1.0, 0, None) == abi.ERR_TOO_LARGE  # delta pass: 2^32 threads
+    assert lib.fused_mha_backward_workspace_bytes(1, 1 << 17, 128, 128) == 0
+    assert lib.fused_mha_backward_min_workspace_bytes(1, 1 << 17, 128, 128) == 0
 
 
 def test_backward_validation_codes(lib):
@@ -227,6 +234,75 @@ int main() {
 ''')
     inc = os.path.join(abi.ROOT, "flash-attention-v100_amd", "csrc")
     exe = tmp_path / "check_block_map"
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-I", inc, str(src), "-o", str(exe)])
+    assert subprocess.check_output([str(exe)]).decode().strip() == "ok"
+
+
+def test_persistent_schedule_covers_every_block_once_and_balances(tmp_path):
+    """csrc/block_map.h, compiled for the host: the rounds of the persistent work groups visit every block exactly
+    once, a work group's blocks stay on its XCD (block number mod 8), and under causal masking the static
+    schedule is balanced: at the headline and the long-context shape no work group gets more than 3 % above the
+    mean number of tiles."""
+    import os
+    import subprocess
+
+    src = tmp_path / "check_persistent.cpp"
+    src.write_text(r'''
+#include <cstdio>
+#include <vector>
+#include <algorithm>
+#include "block_map.h"
+static int check(int total, int G) {
+  std::vector<int> seen(total, 0);
+  for (int w = 0; w < G; ++w) {
+    int r = 0;
+    if (fmha_persistent_block(0, w, G) >= total) { printf("first round %d %d %d\n", total, G, w); return 1; }
+    int guard = 0;
+    while (r >= 0) {
+      const int lin = fmha_persistent_block(r, w, G);
+      if (lin < 0 || lin >= total) { printf("range %d %d %d %d\n", total, G, w, r); return 1; }
+      if ((lin & 7) != (w & 7) && total > G) { printf("xcd %d %d %d %d\n", total, G, w, r); return 1; }
+      if (seen[lin]++) { printf("twice %d %d %d\n", total, G, lin); return 1; }
+      r = fmha_persistent_next_round(r, w, G, total);
+      if (++guard > total + 2) { printf("no end %d %d %d\n", total, G, w); return 1; }
+    }
+  }
+  for (int lin = 0; lin < total; ++lin) if (!seen[lin]) { printf("missed %d %d %d\n", total, G, lin); return 1; }
+  return 0;
+}
+// tiles per work group under causal masking: slices x bps blocks of `rows` queries, 64-key tiles
+static double imbalance(int slices, int bps, int rows, int G) {
+  const int total = slices * bps;
+  std::vector<long> load(G, 0);
+  for (int w = 0; w < G; ++w)
+    for (int r = 0; r >= 0; r = fmha_persistent_next_round(r, w, G, total)) {
+      int s, b;
+      fmha_slice_and_block(fmha_persistent_block(r, w, G), slices, bps, s, b);
+      const int mblk = bps - 1 - b;  // heavy first
+      load[w] += (long)(mblk + 1) * rows / 64;
+    }
+  long sum = 0, mx = 0;
+  for (long v : load) { sum += v; mx = std::max(mx, v); }
+  return (double)mx * G / sum;
+}
+int main() {
+  for (int G : {8, 64, 256, 304})
+    for (int total = 1; total <= 5 * G + 17; total += (total < 40 ? 1 : 7)) {
+      const int grid = total <= G ? total : G;  // what persistent_grid() launches
+      if (check(total, grid)) return 1;
+    }
+  const double head_fwd = imbalance(64, 16, 256, 256), head_dq = imbalance(64, 32, 128, 256);
+  const double long_fwd = imbalance(16, 64, 256, 256), long_dq = imbalance(16, 128, 128, 256);
+  if (head_fwd > 1.03 || head_dq > 1.03 || long_fwd > 1.03 || long_dq > 1.03) {
+    printf("imbalance %.3f %.3f %.3f %.3f\n", head_fwd, head_dq, long_fwd, long_dq);
+    return 1;
+  }
+  puts("ok");
+  return 0;
+}
+''')
+    inc = os.path.join(abi.ROOT, "flash-attention-v100_amd", "csrc")
+    exe = tmp_path / "check_persistent"
     subprocess.check_call(["g++", "-O1", "-std=c++17", "-I", inc, str(src), "-o", str(exe)])
     assert subprocess.check_output([str(exe)]).decode().strip() == "ok"
 

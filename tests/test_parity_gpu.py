@@ -367,6 +367,110 @@ def test_hip_graph_capture_and_replay():
         assert _err(replayed[0], o_ref) <= O_TOL
 
 
+SPILL_CASES = [  # B, H, N, D, causal
+    (1, 2, 64, 128, True), (2, 3, 333, 64, True), (1, 2, 70, 128, False), (1, 2, 40, 64, True),
+    (1, 2, 1031, 128, True), (2, 4, 512, 64, False), (1, 20, 384, 128, True), (1, 9, 1500, 64, False),
+]
+
+
+@pytest.mark.parametrize("B,H,N,D,causal", SPILL_CASES)
+def test_spill_and_recompute_backward_agree(lib, B, H, N, D, causal):
+    """The backward has two paths, chosen by the size of the workspace: with room for the dS tiles the dK/dV pass
+    spills them and the dQ pass is one GEMM; with the minimum workspace the dQ pass recomputes S and dP.  dK and
+    dV come from the same arithmetic (bit-equal); dQ sums the same products tile by tile (equal to rounding);
+    both match the oracle."""
+    scale = 1.0 / math.sqrt(D)
+    q, k, v, do = ao.make_inputs(B, N, H, D, seed=5 * N + D)
+    print(f"spill/recompute B{B} H{H} N{N} D{D} causal={causal}", flush=True)
+    assert lib.fused_mha_backward_workspace_bytes(B, H, N, D) > lib.fused_mha_backward_min_workspace_bytes(B, H, N, D)
+    qg, kg, vg, dog = (t.cuda() for t in (q, k, v, do))
+    out, lse = abi.forward(lib, qg, kg, vg, scale, causal)
+    dq_s, dk_s, dv_s, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal)
+    dq_p, dk_p, dv_p, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal, split=True)
+    dq_r, dk_r, dv_r, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal, min_workspace=True)
+    torch.cuda.synchronize()
+    assert torch.equal(dk_s, dk_r) and torch.equal(dv_s, dv_r)
+    assert torch.equal(dq_s, dq_p) and torch.equal(dk_s, dk_p) and torch.equal(dv_s, dv_p)  # per-pass entry points
+    assert (dq_s.float() - dq_r.float()).abs().max().item() <= 2e-3
+    dq_ref, dk_ref, dv_ref = ao.attention_backward(q, k, v, do, scale, causal)
+    for got in (dq_s, dq_r):
+        assert _err(got, dq_ref) <= G_TOL
+    assert _err(dk_s, dk_ref) <= G_TOL and _err(dv_s, dv_ref) <= G_TOL
+    assert torch.isfinite(dq_s).all()
+
+
+def _forward_oracle_in_row_chunks(q, k, v, scale, causal, chunk=2048):
+    """attention_oracle.attention_forward for ONE (batch, head) slice, evaluated in chunks of query rows so that
+    the score matrix in memory is chunk x N (fp32) instead of N x N; same formulas (test.py:13-26)."""
+    N = q.shape[0]
+    outs, lses = [], []
+    for r0 in range(0, N, chunk):
+        r1 = min(N, r0 + chunk)
+        nk = r1 if causal else N  # keys past the chunk's last row are masked for all of its rows
+        s = (q[r0:r1].float() @ k[:nk].float().t()) * scale
+        if causal:
+            rows = torch.arange(r0, r1).unsqueeze(1)
+            s = s.masked_fill(torch.arange(nk).unsqueeze(0) > rows, float("-inf"))
+        lses.append(torch.logsumexp(s, dim=-1))
+        outs.append(torch.softmax(s, dim=-1) @ v[:nk].float())
+    return torch.cat(outs), torch.cat(lses)
+
+
+def test_long_context_forward_all_heads(lib):
+    """B1 H16 N16384 D128 causal: O and lse of every head against the oracle (in row chunks: a whole head's score
+    matrix would be 1 GiB), not only of the three heads whose backward is checked."""
+    B, H, N, D, causal = 1, 16, 16384, 128, True
+    scale = 1.0 / math.sqrt(D)
+    torch.set_num_threads(16)
+    q, k, v, _ = ao.make_inputs(B, N, H, D, seed=20, zero_tail_rows=32)
+    out, lse = abi.forward(lib, q.cuda(), k.cuda(), v.cuda(), scale, causal)
+    torch.cuda.synchronize()
+    out, lse = out.cpu(), lse.cpu()
+    # the chunked evaluation is the oracle's: same numbers on a head small enough for both
+    o_small, l_small = _forward_oracle_in_row_chunks(q[0, :3000, 0], k[0, :3000, 0], v[0, :3000, 0], scale, causal, 512)
+    o_ref, l_ref = ao.attention_forward(q[:, :3000, :1], k[:, :3000, :1], v[:, :3000, :1], scale, causal)
+    assert (o_small - o_ref[0, :, 0]).abs().max().item() <= 1e-5 and (l_small - l_ref[0, 0]).abs().max().item() <= 1e-4
+    for h in range(H):
+        o_ref, l_ref = _forward_oracle_in_row_chunks(q[0, :, h], k[0, :, h], v[0, :, h], scale, causal)
+        eo = (out[0, :, h].float() - o_ref.half().float()).abs().max().item()
+        el = (lse[0, h] - l_ref).abs().max().item()
+        print(f"long context head {h}: O {eo:.2e} lse {el:.2e}", flush=True)
+        assert eo <= O_TOL and el <= LSE_TOL
+
+
+def test_extension_takes_caller_supplied_outputs():
+    """ext.fwd with out_ and ext.bwd with dq_, dk_, dv_ supplied by the caller (reference
+    kernel/fused_mha_api.cpp:49-58, 125-153): the results land in those tensors, equal to the ones the extension
+    allocates itself, and nothing depends on what the tensors held (NaN here; the reference needs dq zero-filled)."""
+    import flash_attn_v100_cuda as ext
+
+    B, H, N, D, causal = 2, 3, 300, 128, True
+    scale = 1.0 / math.sqrt(D)
+    q, k, v, do = ao.make_inputs(B, N, H, D, seed=91)
+    qg, kg, vg, dog = (t.cuda() for t in (q, k, v, do))
+    out0, lse0 = ext.fwd(qg, kg, vg, None, scale, causal)
+    mine = torch.full_like(qg, float("nan"))
+    out1, lse1 = ext.fwd(qg, kg, vg, mine, scale, causal)
+    torch.cuda.synchronize()
+    assert out1.data_ptr() == mine.data_ptr()
+    assert torch.equal(mine, out0) and torch.equal(lse1, lse0)
+    o_ref, _ = ao.attention_forward(q, k, v, scale, causal)
+    assert _err(mine, o_ref) <= O_TOL
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ext.fwd(qg, kg, vg, torch.empty(B, H, N, D, dtype=torch.float16, device="cuda").transpose(1, 2), scale, causal)
+    with pytest.raises(RuntimeError):
+        ext.fwd(qg, kg, vg, torch.empty(B, N, H, D, dtype=torch.float32, device="cuda"), scale, causal)
+
+    dq0, dk0, dv0 = ext.bwd(dog, qg, kg, vg, out0, lse0, None, None, None, scale, causal)
+    grads = [torch.full_like(qg, float("nan")) for _ in range(3)]
+    dq1, dk1, dv1 = ext.bwd(dog, qg, kg, vg, out0, lse0, grads[0], grads[1], grads[2], scale, causal)
+    torch.cuda.synchronize()
+    assert [t.data_ptr() for t in (dq1, dk1, dv1)] == [t.data_ptr() for t in grads]
+    assert torch.equal(grads[0], dq0) and torch.equal(grads[1], dk0) and torch.equal(grads[2], dv0)
+    dq_ref, dk_ref, dv_ref = ao.attention_backward(q, k, v, do, scale, causal)
+    assert _err(grads[0], dq_ref) <= G_TOL and _err(grads[1], dk_ref) <= G_TOL and _err(grads[2], dv_ref) <= G_TOL
+
+
 def test_errors_on_gpu():
     from flash_attn_v100 import flash_attn_func
 
