@@ -38,6 +38,7 @@
 #include "fused_mha.h"
 #include "block_map.h"
 
+
 // Backward workspace of fused_mha_backward_noalloc (delta and lse*log2(e), fp32
 // (batch, head, n) each): lives in the code object, one copy per GPU, so that
 // entry point never allocates.  Host code must not use this name as an address;
@@ -326,6 +327,7 @@ constexpr int kFwdWaves = 8;
 constexpr int kFwdThreads = kFwdWaves * 64;
 constexpr int kFwdBlockQ = kFwdWaves * kResident;
 constexpr int kRing = 3;
+constexpr int kFwdBlockKernelMaxN = 1024;  // D = 64, causal: longest sequence the one-block kernel takes
 
 // The kernel is persistent: the launch has one work group per CU (fewer for small
 // problems) and each walks its own list of blocks (PersistentBlocks).  While a block's
@@ -657,6 +659,233 @@ fmha_fwd_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, cons
   // orders inside the loop, so no register shuffling at branch merges.
   if (first_group) run(IntTag<0>{});
   else run(IntTag<1>{});
+}
+
+// The forward with one block per work group (no persistence, output staged in the rings once the
+// block is done, fragment reads scheduled by hints): with D = 64 it needs few enough registers
+// and little enough LDS (48 KiB) for two work groups per CU, which the persistent kernel does not.
+// The launcher uses it for D = 64 when that matters more than the persistent kernel's balancing
+// and prefetching: without causal masking (all blocks weigh the same) and for short sequences.
+template <int D, bool CAUSAL>
+__global__ void __launch_bounds__(kFwdThreads, 1)
+fmha_fwd_block_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
+                Strides qs, Strides ks, Strides vs, half_t* __restrict__ O, float* __restrict__ LSE, int H, int N,
+                int nmb, float c, int negate_q) {
+  using G = TileGeom<D>;
+  using T = SwzTile<D>;
+  constexpr int kIPW = T::kInstrs / kFwdWaves;  // copy instructions per wave per tile
+  // K ring then V ring, kRing slots each.  The copies into the ring are inline
+  // asm (see copy16), so slots can be addressed at run time.
+  __shared__ __attribute__((aligned(1024))) char smem[2 * kRing * T::kBytes];
+  char* const k_ring = smem;
+  char* const v_ring = smem + kRing * T::kBytes;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = lane & 31, hh = lane >> 5;
+  int bh, mb;
+  slice_and_block(nmb, bh, mb);
+  const int mblk = CAUSAL ? nmb - 1 - mb : mb;  // heavy blocks first
+  const int b = bh / H, h = bh - b * H;
+  const int rs = H * D;  // O is dense
+  const long head_off = ((long)b * N * H + h) * D;
+  const half_t* Qb = Q + b * qs.b + (long)h * qs.h;
+  const half_t* Kb = K + b * ks.b + (long)h * ks.h;
+  const half_t* Vb = V + b * vs.b + (long)h * vs.h;
+
+  const int m0 = mblk * kFwdBlockQ;
+  const int q0w = m0 + wave * kResident;
+  const int qi = q0w + i;
+
+  // nt: tiles the block streams; ntw: tiles this wave has unmasked keys in.
+  int nt = (N + kTile - 1) / kTile;
+  int ntw = nt;
+  if (CAUSAL) {
+    nt = min(nt, (min(m0 + kFwdBlockQ, N) - 1) / kTile + 1);
+    ntw = min(nt, (min(q0w + kResident, N) - 1) / kTile + 1);
+    if (q0w >= N) ntw = 0;
+  }
+
+  // this wave's share of every tile copy
+  int c_row[kIPW], c_kgoff[kIPW], c_vgoff[kIPW], c_blk[kIPW];
+#pragma unroll
+  for (int u = 0; u < kIPW; ++u) {
+    const int t = wave * kIPW + u;
+    copy_src<D>(t, lane, ks.n, c_row[u], c_kgoff[u]);
+    copy_src<D>(t, lane, vs.n, c_row[u], c_vgoff[u]);
+    c_blk[u] = t * 1024;
+  }
+  auto copy_tile = [&](const half_t* src, int src_rs, const int (&goff)[kIPW], char* dst, int tile_idx)
+                       __attribute__((always_inline)) {
+    const int row0 = tile_idx * kTile;
+    const half_t* tp = src + (long)row0 * src_rs;  // wave-uniform
+    if (row0 + kTile <= N) {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) copy16(tp, goff[u], dst + c_blk[u]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < kIPW; ++u) {  // rows past the end re-read row N-1
+        const int back = max(row0 + c_row[u] - (N - 1), 0);
+        copy16(tp, goff[u] - back * src_rs * 2, dst + c_blk[u]);
+      }
+    }
+  };
+
+  copy_tile(Kb, ks.n, c_kgoff, k_ring, 0);
+  if (nt > 1) copy_tile(Kb, ks.n, c_kgoff, k_ring + T::kBytes, 1);
+  copy_tile(Vb, vs.n, c_vgoff, v_ring, 0);
+
+  h8 qf[G::kKSteps];
+  {
+    const half_t* qp = Qb + (long)min(qi, N - 1) * qs.n + hh * 8;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+      qf[kk] = *reinterpret_cast<const h8*>(qp + kk * 16);
+      if (negate_q) qf[kk] = -qf[kk];
+    }
+  }
+
+  int k_off[2], v_off[2];
+  swz_rows_off<D>(lane, k_off);
+  swz_cols_off<D>(lane, v_off);
+
+  f16v o[G::kDBlocks];
+#pragma unroll
+  for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  f16v s[2];   // scores of the tile in flight
+  h8 pf[4];    // its probabilities, fp16, B-operand order
+
+  auto scores = [&](const char* Kl, int t) __attribute__((always_inline)) {
+    if (t >= ntw) return;
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[rb][r] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < G::kKSteps; ++kk) {
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) s[rb] = mfma(swz_rows<D>(Kl, rb, kk, k_off), qf[kk], s[rb]);
+    }
+    // LDS reads run kLead MFMAs ahead of their use.
+    constexpr int kN = 2 * G::kKSteps, kLead = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
+#pragma unroll
+    for (int n = 0; n < kN - kLead; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
+  };
+  auto softmax = [&](int t) __attribute__((always_inline)) {
+    if (t < 0 || t >= ntw) return;
+    const int key0 = t * kTile;
+    if ((CAUSAL && key0 + kTile - 1 > q0w) || (key0 + kTile > N)) {
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          int key = key0 + acc_row(rb, r, hh);
+          if ((CAUSAL && key > qi) || key >= N) s[rb][r] = -INFINITY;
+        }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[rb][r]);
+    mx = fmaxf(mx, other_half(mx));
+    const float m_new = fmaxf(m_run, mx);
+    if (__builtin_amdgcn_ballot_w64((m_new - m_run) * c > kRescaleLog2) != 0) {
+      const float alpha = fast_exp2((m_run - m_new) * c);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[db][r] *= alpha;
+    }
+    // Row sums with plain fp32 adds: the dot-product instructions share the
+    // matrix pipeline and stall behind the other wave's MFMAs.
+    const float mc = m_run * c;
+    float l0 = 0.f, l1 = 0.f;
+#pragma unroll
+    for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const float p0 = fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + e], c, -mc));
+        const float p1 = fast_exp2(fmaf(s[c16 >> 1][(c16 & 1) * 8 + e + 1], c, -mc));
+        pf[c16][e] = (half_t)p0;
+        pf[c16][e + 1] = (half_t)p1;
+        l0 += p0;
+        l1 += p1;
+      }
+    }
+    l_run += l0 + l1;
+  };
+  auto accumulate = [&](const char* Vl, int t) __attribute__((always_inline)) {
+    if (t < 0 || t >= ntw) return;
+#pragma unroll
+    for (int c16 = 0; c16 < 4; ++c16) {
+#pragma unroll
+      for (int db = 0; db < G::kDBlocks; ++db) o[db] = mfma(swz_cols<D>(Vl, c16, db, v_off), pf[c16], o[db]);
+    }
+    // LDS reads (two per MFMA) run kLead MFMAs ahead of their use.
+    constexpr int kN = 4 * G::kDBlocks, kLead = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead, 0);
+#pragma unroll
+    for (int n = 0; n < kN - kLead; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
+  };
+
+  const bool first_group = wave < kFwdWaves / 2;
+  // Everything issued so far (Q rows, first copies) is waited for here, once,
+  // so that no wait for a register load is left to be placed inside the loop,
+  // where it would also wait for the copies in flight.
+  wait_vm<0>();
+  // Iteration j: K(j) sits in K slot j % 3, V(j-1) in V slot (j-1) % 3; K(j+2)
+  // is copied into K slot (j+2) % 3 and V(j+1) into V slot (j+1) % 3.
+  auto run = [&](auto group_tag) __attribute__((always_inline)) {
+    constexpr bool kFirst = decltype(group_tag)::value == 0;
+    int s0 = 0, s1 = 1, s2 = 2;  // j % 3, (j+1) % 3, (j+2) % 3
+    for (int j = 0; j <= nt; ++j) {
+      // K(j) and V(j-1) were issued two iterations ago; what the previous
+      // iteration issued (K(j+1), V(j)) may still be in flight.
+      if (j + 1 < nt) wait_vm<2 * kIPW>();
+      else if (j < nt) wait_vm<kIPW>();
+      else wait_vm<0>();
+      block_barrier();
+      if (j + 2 < nt) copy_tile(Kb, ks.n, c_kgoff, k_ring + s2 * T::kBytes, j + 2);
+      if (j + 1 < nt) copy_tile(Vb, vs.n, c_vgoff, v_ring + s1 * T::kBytes, j + 1);
+      const char* Kl = k_ring + s0 * T::kBytes;
+      const char* Vl = v_ring + s2 * T::kBytes;
+      if (kFirst) {
+        accumulate(Vl, j - 1);
+        if (j < nt) { scores(Kl, j); softmax(j); }
+      } else {
+        softmax(j - 1);
+        accumulate(Vl, j - 1);
+        if (j < nt) scores(Kl, j);
+      }
+      const int t = s0; s0 = s1; s1 = s2; s2 = t;
+    }
+  };
+  // Each group runs its own copy of the loop: no joins between the two
+  // orders inside the loop, so no register shuffling at branch merges.
+  if (first_group) run(IntTag<0>{});
+  else run(IntTag<1>{});
+
+  const float l_tot = l_run + other_half(l_run);
+  const float inv = 1.f / l_tot;
+  static_assert(kFwdWaves * StageGeom<D>::kBytes <= 2 * kRing * T::kBytes, "the output staging tiles fit the rings");
+  block_barrier();  // every wave is done with the rings: they become the staging tiles
+  store_resident<D>(O + head_off, rs, q0w, N, o, inv, lane, smem + wave * StageGeom<D>::kBytes);
+  if (hh == 0 && qi < N) LSE[((long)b * H + h) * N + qi] = (m_run * c + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }
 
 // ---------------------------------------------------------------------------
@@ -1583,6 +1812,14 @@ int launch_forward(const void* q, const void* k, const void* v, Strides qs, Stri
   // scale == 0 would turn the masked scores (-inf) into NaN when multiplied; a
   // tiny positive factor gives the same uniform softmax and keeps -inf * c = -inf.
   const float c = fmaxf(fabsf(scale) * kLog2e, 1e-30f);
+  if constexpr (D == 64) {
+    if (!CAUSAL || n <= kFwdBlockKernelMaxN) {  // see fmha_fwd_block_kernel
+      const hipError_t rc = launch(fmha_fwd_block_kernel<D, CAUSAL>, (unsigned)total, kFwdThreads, stream,
+                                   (const half_t*)q, (const half_t*)k, (const half_t*)v, qs, ks, vs, (half_t*)o,
+                                   (float*)lse, head, n, nmb, c, scale < 0.f ? 1 : 0);
+      return rc == hipSuccess ? FUSED_MHA_OK : FUSED_MHA_ERR_LAUNCH;
+    }
+  }
   const hipError_t rc = launch(fmha_fwd_kernel<D, CAUSAL>, grid, kFwdThreads, stream, (const half_t*)q,
                                (const half_t*)k, (const half_t*)v, qs, ks, vs, (half_t*)o, (float*)lse, head, n, nmb, total, c,
                                scale < 0.f ? 1 : 0);
