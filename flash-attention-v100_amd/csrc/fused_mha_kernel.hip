@@ -72,6 +72,25 @@ __device__ __forceinline__ f16v mfma(h8 a, h8 b, f16v c) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// dS for two neighbouring positions: fp16(-p.lo * x0) and fp16(-p.hi * x1), the products in fp32, as
+// two mixed-precision FMAs that read the fp16 halves of p directly (the same bits as converting p to
+// fp32, multiplying and converting back, in 2 instructions instead of 5).
+typedef unsigned u4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ unsigned neg_mul_to_f16x2(unsigned p_pair, float x0, float x1) {
+  unsigned r = 0;
+  asm("v_fma_mixlo_f16 %0, %1, -%2, 0 op_sel_hi:[1,0,0]" : "+v"(r) : "v"(p_pair), "v"(x0));
+  asm("v_fma_mixhi_f16 %0, %1, -%2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(r) : "v"(p_pair), "v"(x1));
+  return r;
+}
+// y[.] = fp16(-p[.] * x[.]) for the 8 values of one B-operand fragment
+__device__ __forceinline__ h8 neg_mul_to_f16x8(h8 p, const float* x) {
+  const u4v pp = __builtin_bit_cast(u4v, p);
+  u4v r;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) r[j] = neg_mul_to_f16x2(pp[j], x[2 * j], x[2 * j + 1]);
+  return __builtin_bit_cast(h8, r);
+}
+
 // Combine a value with the one held by the lane 32 positions away.
 __device__ __forceinline__ float other_half(float x) {
   int xi = __float_as_int(x);
@@ -297,6 +316,14 @@ __device__ __forceinline__ void wait_vm_tiles(int later) {
 }
 template <int V>
 struct IntTag { static constexpr int value = V; };
+
+// 16 bytes per lane to p + kOffset bytes, with the non-temporal hint (data that is read once, by a later
+// kernel).  Inline asm because the compiler keeps the hint only on the first of several stores that share
+// a base address; like the tile copies it is therefore invisible to the compiler's wait counts.
+template <int kOffset>
+__device__ __forceinline__ void store16_stream(half_t* p, h8 v, IntTag<kOffset>) {
+  asm volatile("global_store_dwordx4 %0, %1, off offset:%2 nt" : : "v"(p), "v"(v), "n"(kOffset) : "memory");
+}
 
 // Element strides of a (batch, n, head, d) tensor whose last dimension is
 // contiguous.  The dense layout of reference kernel/fused_mha_kernel.cu:57-59 is
@@ -1162,11 +1189,11 @@ fmha_bwd_dq_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K, c
         for (int rb = 0; rb < 2; ++rb) {
           const h8 p0 = *reinterpret_cast<const h8*>(pr + rb * 2048);
           const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 1024);
+          float xr[16];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            y[rb * 2][e] = (half_t)(-(float)p0[e] * x[rb][e]);
-            y[rb * 2 + 1][e] = (half_t)(-(float)p1[e] * x[rb][8 + e]);
-          }
+          for (int e = 0; e < 16; ++e) xr[e] = x[rb][e];
+          y[rb * 2] = neg_mul_to_f16x8(p0, xr);
+          y[rb * 2 + 1] = neg_mul_to_f16x8(p1, xr + 8);
         }
 #pragma unroll
         for (int c16 = 0; c16 < 4; ++c16) {
@@ -1449,9 +1476,9 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
       for (int r = 0; r < 16; ++r) x[rb][r] = 0.f;
     for (int it = 0; it <= n_it; ++it) {
-      // SPILL: the stores of dS are issued before this iteration's tile copies, so that the
-      // wait at the top of the next iteration (everything but the newest copies) covers them
-      // whatever order stores and copies complete in.
+      // SPILL: this wave issues its tile copies and, after the second GEMM, the four stores of dS.  The wait
+      // at the top of the next iteration leaves at most as many operations in flight as those stores, the
+      // newest: every copy issued so far has then landed, whatever order stores and copies complete in.
       if (SPILL) step_wait(it);
       else step_sync(it);
       const bool prev_active = it >= 1 && tile_active(it - 1);
@@ -1462,11 +1489,11 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
         for (int rb = 0; rb < 2; ++rb) {
           const h8 p0 = *reinterpret_cast<const h8*>(pr + rb * 2048);
           const h8 p1 = *reinterpret_cast<const h8*>(pr + rb * 2048 + 1024);
+          float xr[16];
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            y[rb * 2][e] = (half_t)(-(float)p0[e] * x[rb][e]);
-            y[rb * 2 + 1][e] = (half_t)(-(float)p1[e] * x[rb][8 + e]);
-          }
+          for (int e = 0; e < 16; ++e) xr[e] = x[rb][e];
+          y[rb * 2] = neg_mul_to_f16x8(p0, xr);
+          y[rb * 2 + 1] = neg_mul_to_f16x8(p1, xr + 8);
         }
         if (SPILL) {
           if (k0w + kResident > N && ki >= N) {  // keys past the end contribute nothing to dQ
@@ -1475,16 +1502,20 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 #pragma unroll
               for (int e = 0; e < 8; ++e) y[c16][e] = (half_t)0.f;
           }
-          const int t = t_begin + it - 1;  // the query tile
-          half_t* dst = ds_lane + (long)(t >> 1) * np * 128 + (t & 1) * 2048;
-#pragma unroll
-          for (int c16 = 0; c16 < 4; ++c16) {
-            __builtin_nontemporal_store(y[c16], reinterpret_cast<h8*>(dst + c16 * 512));  // read once, later
-          }
         }
       }
       if (SPILL && it + 2 < n_it) copy_tiles(it + 2);
       if (prev_active) gemm2(q_ring + ((it - 1) & 3) * T::kBytes, y);
+      if (SPILL && prev_active) {
+        // dS(it - 1) leaves here, between the two GEMMs and away from the tile copies, which all waves issue
+        // right after the barrier: the stores go through the same path and would queue behind them.
+        const int t = t_begin + it - 1;  // the query tile
+        half_t* dst = ds_lane + (long)(t >> 1) * np * 128 + (t & 1) * 2048;
+        store16_stream(dst, y[0], IntTag<0>{});
+        store16_stream(dst, y[1], IntTag<1024>{});
+        store16_stream(dst, y[2], IntTag<2048>{});
+        store16_stream(dst, y[3], IntTag<3072>{});
+      }
       if (it < n_it && tile_active(it)) {
         const char* Gl = g_ring + (it % 3) * T::kBytes;
         const char* Sl = st_ring + (it % 3) * kStBytes + st_off;
