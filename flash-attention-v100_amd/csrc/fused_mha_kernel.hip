@@ -127,12 +127,14 @@ struct StageGeom {
 template <int D>
 __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long row_stride, int row0, int n,
                                                const f16v (&acc)[TileGeom<D>::kDBlocks], float mul, int lane,
-                                               char* __restrict__ stage, int my_row = -1) {
+                                               char* __restrict__ stage, int my_row = -1,
+                                               int upper_off = 16 * StageGeom<D>::kPitch) {
   // my_row: the row (0..31, relative to row0) this lane's column of the accumulator belongs
-  // to, when that is not lane & 31 (see fmha_bwd_dq_spill_kernel)
+  // to, when that is not lane & 31; upper_off: where rows 16..31 are staged, relative to `stage`,
+  // when the staging tile is not contiguous (see fmha_bwd_dq_spill_kernel for both)
   constexpr int kPitch = StageGeom<D>::kPitch;
   const int i = my_row < 0 ? (lane & 31) : my_row, hh = lane >> 5;
-  char* mine = stage + i * kPitch + hh * 8;
+  char* mine = stage + (i & 15) * kPitch + (i >> 4) * upper_off + hh * 8;
 #pragma unroll
   for (int db = 0; db < TileGeom<D>::kDBlocks; ++db) {
 #pragma unroll
@@ -150,8 +152,9 @@ __device__ __forceinline__ void store_resident(half_t* __restrict__ base, long r
 #pragma unroll
   for (int pass = 0; pass < kResident / kRowsPerPass; ++pass) {
     const int r = pass * kRowsPerPass + r_in;
-    const h4 lo = *reinterpret_cast<const h4*>(stage + r * kPitch + ch * 16);
-    const h4 hi = *reinterpret_cast<const h4*>(stage + r * kPitch + ch * 16 + 8);
+    const char* src = stage + (r & 15) * kPitch + (r >> 4) * upper_off + ch * 16;
+    const h4 lo = *reinterpret_cast<const h4*>(src);
+    const h4 hi = *reinterpret_cast<const h4*>(src + 8);
     const h8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     if (row0 + r < n) *reinterpret_cast<h8*>(base + (long)(row0 + r) * row_stride + ch * 8) = v;
   }
@@ -1543,63 +1546,72 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 // ---------------------------------------------------------------------------
 // Backward, dQ from spilled dS: dQ = scale * dS K, one GEMM, for callers whose
 // workspace holds the dS tiles fmha_bwd_dkdv_kernel<.., SPILL> wrote (layout there).
-// A block is 128 queries; of the 8 waves, wave w owns the 32 queries qb = w & 3 of the
-// block and half of the features (w >> 2), and computes per 64 keys
+// A block is P = 1 or 2 of the 128-query panels of the workspace; computing wave
+// w of 4 P owns its 32 queries and computes per 64 keys
 //     dQ^T[d][q] += K^T[d][key] dS^T[key][q]
 // with both operands read transposed out of LDS (the K tile as everywhere else, the
 // dS tile as its 1 KiB pieces), so the order of the keys inside a 16-key step is the
 // same for both.
-// The kernel is bound by reading dS from HBM once, so what matters is that the stream
-// of tile copies never stops: the launch is persistent (PersistentBlocks) and the tiles
-// of a work group's blocks form ONE sequence that runs through the rings without regard
-// to block boundaries; an output block leaves through staging tiles of its own while
-// the copies of the next blocks' tiles are already in flight.  The 16 KiB dS tiles go
-// through a 5-slot ring, four tiles ahead, copied by waves 0-3 only; the K tiles (L2
-// hits) through a 3-slot ring, two ahead, copied by waves 4-7 only.  A wave's copies
-// complete in order, so a wave that issued both would have to wait for young dS copies
-// whenever it needs an older K tile.
+// What bounds the kernel is the path that copies tiles into LDS (64 bytes per clock and
+// CU at best), then HBM (dS is read once):
+//   * with P = 2 a K tile serves 256 queries, so per 32 KiB of dS only 16 KiB of K go through it (P = 1 is
+//     for launches with too few blocks to balance otherwise);
+//   * four more waves do nothing but copy, two the dS tiles (half of the pieces each) and two the
+//     K tiles: issuing a tile's copy instructions holds a wave for about as long as its
+//     share of the MFMAs takes; and a wave's copies complete in order, so a wave that
+//     issued both kinds would wait for young dS copies whenever it needs an older K tile;
+//   * the launch is persistent (PersistentBlocks) and the tiles of a work group's blocks
+//     form ONE sequence that runs through the rings without regard to block boundaries;
+//     an output block leaves through staging tiles of its own while the copies of the
+//     next blocks' tiles are already in flight.  Both rings are filled two tiles ahead: behind the dS copies
+//     that a CU has in flight, a K tile takes as long to arrive as they do, L2 hit or not;
+//   * the LDS is full with that, so the epilogue stages a wave's output rows in the 4 KiB of the block's last dS
+//     tile that hold the wave's own queries and that no other wave reads.
 // The queries of a chunk sit in the order the dK/dV pass's registers held them (bits
 // 2 and 3 of the position inside 16 swapped); the epilogue puts the rows back in place.
 // (formula: reference kernel/fused_mha_kernel.cu:680-683.)
 // ---------------------------------------------------------------------------
-constexpr int kDsWaves = 8;
-constexpr int kDsThreads = kDsWaves * 64;
-constexpr int kDsBlockQ = 128;
-constexpr int kDsRingS = 5;   // dS tiles
+constexpr int kDsCopyWaves = 4;    // waves that only copy tiles: two for dS, two for K
+constexpr int kDsPanelQ = 128;     // queries per panel of the workspace
+constexpr int kDsRingS = 3;   // dS tiles
 constexpr int kDsRingK = 3;   // K tiles
-constexpr int kDsTileBytes = kTile * kDsBlockQ * 2;
+constexpr int kDsPanelTileBytes = kTile * kDsPanelQ * 2;
 constexpr int kDsStageD = 32;          // features staged at a time in the epilogue
+constexpr int ds_threads(int panels) { return (4 * panels + kDsCopyWaves) * 64; }
 
-template <int D, bool CAUSAL>
-__global__ void __launch_bounds__(kDsThreads, 1)
+template <int D, bool CAUSAL, int kDsPanels>
+__global__ void __launch_bounds__(ds_threads(kDsPanels), 1)
 fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t* __restrict__ dS, int np,
                          half_t* __restrict__ dQ, int H, int N, int nqb, int total, float scale) {
   using T = SwzTile<D>;             // K tile: 64 keys x D features
-  constexpr int kCopyWaves = kDsWaves / 2;
-  constexpr int kKIPW = T::kInstrs / kCopyWaves;           // K copies per K-copying wave and tile
-  constexpr int kSIPW = (kDsTileBytes / 1024) / kCopyWaves;  // dS copies per dS-copying wave and tile
-  constexpr int kDBW = D / 64;      // 32-feature blocks per wave
-  constexpr int kStageBytes = StageGeom<kDsStageD>::kBytes;
-  __shared__ __attribute__((aligned(1024))) char smem[kDsRingS * kDsTileBytes + kDsRingK * T::kBytes + kDsWaves * kStageBytes];
+  constexpr int kKIPW = T::kInstrs / 2;              // K copies per K-copying wave and tile
+  constexpr int kDsWaves = 4 * kDsPanels;            // computing waves
+  constexpr int kDsBlockQ = kDsPanels * kDsPanelQ;
+  constexpr int kDsTileBytes = kDsPanels * kDsPanelTileBytes;
+  constexpr int kSIPW = kDsTileBytes / 1024 / 2;     // dS copies per dS-copying wave and tile: half of the pieces
+  constexpr int kDB = D / 32;       // 32-feature blocks
+  static_assert(16 * StageGeom<kDsStageD>::kPitch <= 2048, "half a staging tile must fit into two dS pieces");
+  __shared__ __attribute__((aligned(1024))) char smem[kDsRingS * kDsTileBytes + kDsRingK * T::kBytes];
   char* const s_ring = smem;
   char* const k_ring = smem + kDsRingS * kDsTileBytes;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int qb = wave & 3, dh = wave >> 2;
-  const bool copies_k = wave >= kCopyWaves;
-  const int cw = wave & (kCopyWaves - 1);
+  const bool computes = wave < kDsWaves;             // then two waves that copy dS and two that copy K
+  const int qb = wave & (kDsWaves - 1);              // computing wave: its 32 queries of the block
+  const bool copies_k = wave >= kDsWaves + 2;
+  const int cw = wave & 1;                           // copying wave: which half of its tensor's copies
   const int i = lane & 31;
-  char* const stage = smem + kDsRingS * kDsTileBytes + kDsRingK * T::kBytes + wave * kStageBytes;
   const int rs = H * D;  // dQ is dense
   const int nt_all = (N + kTile - 1) / kTile;
+  const int n_panels = np / kDsPanelQ;
   const int slices = total / nqb;
   const PersistentBlocks pb{total};
 
   // A position in the work group's sequence of tiles: block (round, number), tile j of its nt.
   struct Cursor {
     int round, lin, j, nt, mblk;
-    const half_t* base;  // the block's dS panel (consumer and dS copies) or the slice's K rows (K copies)
+    const half_t* base;  // dS copies: this wave's pieces of the block's tile 0; K copies: the slice's K rows
     long out_off;        // consumer: element offset of the slice in dQ
   };
   auto open = [&](int round, bool for_k) __attribute__((always_inline)) {
@@ -1611,8 +1623,13 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
     c.mblk = CAUSAL ? nqb - 1 - mb : mb;  // heavy blocks first
     const int b = bh / H, h = bh - b * H;
     c.j = 0;
-    c.nt = CAUSAL ? min(nt_all, 2 * c.mblk + 2) : nt_all;
-    c.base = for_k ? K + b * ks.b + (long)h * ks.h : dS + (((long)bh * nqb + c.mblk) * np) * kDsBlockQ;
+    c.nt = CAUSAL ? min(nt_all, 2 * kDsPanels * (c.mblk + 1)) : nt_all;
+    // the pieces of a dS-copying wave: with two panels per block one whole panel (the last block of a sequence
+    // may have one panel only: the second wave then re-reads the first), else one half of the panel
+    const int panel = kDsPanels == 2 ? min(2 * c.mblk + cw, n_panels - 1) : c.mblk;
+    const int first_piece = kDsPanels == 2 ? 0 : cw * kSIPW;
+    c.base = for_k ? K + b * ks.b + (long)h * ks.h
+                   : dS + (((long)bh * n_panels + panel) * np) * kDsPanelQ + first_piece * 512;
     c.out_off = ((long)b * N * H + h) * D;
     return c;
   };
@@ -1628,11 +1645,11 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
     int bh, mb;
     fmha_slice_and_block(pb.lin(r), slices, nqb, bh, mb);
     const int mblk = CAUSAL ? nqb - 1 - mb : mb;
-    n_tiles += CAUSAL ? min(nt_all, 2 * mblk + 2) : nt_all;
+    n_tiles += CAUSAL ? min(nt_all, 2 * kDsPanels * (mblk + 1)) : nt_all;
   }
 
-  // K copies: this wave's share of a tile (as in the other kernels).  dS copies: piece p = cw * kSIPW + u of
-  // the tile, 1 KiB, lane l fetching 16 bytes.  In memory a piece is [2 halves][32 keys] x 16 bytes; in LDS it
+  // K copies: this wave's half of a tile (as in the other kernels).  dS copies: this wave's kSIPW pieces of
+  // 1 KiB, lane l fetching 16 bytes.  In memory a piece is [2 halves][32 keys] x 16 bytes; in LDS it
   // becomes [32 keys][2 halves] x 16 bytes (rows of 16 queries), and the pieces of odd query chunks land rotated
   // by 128 bytes (LDS offset o holds row-major byte (o - 128) mod 1024), which keeps the two halves of a 32-lane
   // transposing read on different banks.
@@ -1643,18 +1660,17 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
     copy_src<D>(t, lane, ks.n, c_row[u], c_kgoff[u]);
     c_kblk[u] = t * 1024;
   }
-  int c_sgoff[kSIPW];
-#pragma unroll
-  for (int u = 0; u < kSIPW; ++u) {
-    const int piece = cw * kSIPW + u;
-    const int at = (piece & 1) ? (lane - 8) & 63 : lane;  // position (key, half) = (at >> 1, at & 1) of the piece in LDS
-    c_sgoff[u] = piece * 1024 + ((at & 1) * 32 + (at >> 1)) * 16;
+  int c_sgoff[2];  // even and odd pieces; + piece * 1024
+  {
+    const int at = (lane - 8) & 63;  // position (key, half) = (at >> 1, at & 1) in LDS of what lane l fetches of an odd piece
+    c_sgoff[0] = ((lane & 1) * 32 + (lane >> 1)) * 16;
+    c_sgoff[1] = ((at & 1) * 32 + (at >> 1)) * 16;
   }
   auto copy_s = [&](const Cursor& c, int slot) __attribute__((always_inline)) {
-    const half_t* sp = c.base + (long)c.j * (kDsTileBytes / 2);  // wave-uniform
+    const half_t* sp = c.base + (long)c.j * (kDsPanelTileBytes / 2);  // wave-uniform
     char* dst = s_ring + slot * kDsTileBytes + cw * kSIPW * 1024;
 #pragma unroll
-    for (int u = 0; u < kSIPW; ++u) copy16_stream(sp, c_sgoff[u], dst + u * 1024);
+    for (int u = 0; u < kSIPW; ++u) copy16_stream(sp, c_sgoff[u & 1] + u * 1024, dst + u * 1024);
   };
   auto copy_k = [&](const Cursor& c, int slot) __attribute__((always_inline)) {
     const int row0 = c.j * kTile;
@@ -1673,10 +1689,12 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
   };
 
   // LDS offsets of this lane's transposing reads.  K tile: as in the other kernels.  dS tile: key step kc,
-  // read e: key row (kc & 1) * 16 + 8 * e + 4 * hhk + (L >> 2) of the piece [(kc >> 1)][query tile][chunk
+  // read e: key row (kc & 1) * 16 + 8 * e + 4 * hhk + (L >> 2) of the piece [panel][(kc >> 1)][query tile][chunk
   // 2 * (qb & 1) + lane bit 4], 8 bytes at (L & 3) * 8 of its 32-byte row, plus the rotation of odd chunks.
   int c_off[2];
   swz_cols_off<D>(lane, c_off);
+  // the first of this wave's pieces of a dS tile: two adjacent ones per 32 keys
+  const int own_pieces = (qb >> 2) * kDsPanelTileBytes + (((qb >> 1) & 1) * 4 + 2 * (qb & 1)) * 1024;
   int s_off[2][2];
   {
     const int L = lane & 15, odd = (lane >> 4) & 1, hhk = lane >> 5;
@@ -1685,7 +1703,7 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         const int in_piece = (kcl * 16 + 8 * e + 4 * hhk + (L >> 2)) * 32 + (L & 3) * 8;
-        s_off[kcl][e] = ((qb >> 1) * 4 + 2 * (qb & 1) + odd) * 1024 + ((in_piece + odd * 128) & 1023);
+        s_off[kcl][e] = own_pieces + odd * 1024 + ((in_piece + odd * 128) & 1023);
       }
   }
   auto s_frag = [&](const char* tile, int kc) __attribute__((always_inline)) {
@@ -1696,9 +1714,9 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
     return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  f16v acc[kDBW];
+  f16v acc[kDB];
 #pragma unroll
-  for (int db = 0; db < kDBW; ++db)
+  for (int db = 0; db < kDB; ++db)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[db][r] = 0.f;
   // column i of the accumulator is the query at position i of the wave's 32: bits 2 and 3 swapped
@@ -1707,7 +1725,7 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
   constexpr int kAheadS = kDsRingS - 1, kAheadK = kDsRingK - 1;
   // the copying waves run ahead of the sequence: kAhead tiles are issued before the first is used
   Cursor ahead = open(0, copies_k);
-  {
+  if (!computes) {
     const int n_first = min(copies_k ? kAheadK : kAheadS, n_tiles);
     for (int t = 0; t < n_first; ++t) {
       if (copies_k) copy_k(ahead, t);
@@ -1721,34 +1739,48 @@ fmha_bwd_dq_spill_kernel(const half_t* __restrict__ K, Strides ks, const half_t*
   for (int t = 0; t < n_tiles; ++t) {
     // tile t must have landed; the copies of the tiles after it (at most kAhead - 1 of them) may be in flight
     const int later = n_tiles - 1 - t;
-    if (copies_k) wait_vm_tiles<kKIPW, kAheadK - 1>(later);
-    else wait_vm_tiles<kSIPW, kAheadS - 1>(later);
+    if (!computes) {
+      if (copies_k) wait_vm_tiles<kKIPW, kAheadK - 1>(later);
+      else wait_vm_tiles<kSIPW, kAheadS - 1>(later);
+    }
     block_barrier();  // tile t is visible to all; everybody is done with tile t - 1, whose slots are reused now
-    if (ahead.round >= 0) {
+    if (!computes && ahead.round >= 0) {
       if (copies_k) copy_k(ahead, next_k);
       else copy_s(ahead, next_s);
       advance(ahead, copies_k);
     }
-    const int qt = 2 * cur.mblk + (qb >> 1);                                      // this wave's query tile
+    const int qt = 2 * kDsPanels * cur.mblk + (qb >> 1);                          // this wave's query tile
     const int jend = qt >= nt_all ? 0 : (CAUSAL ? min(cur.nt, qt + 1) : cur.nt);  // tiles this wave takes part in
-    if (cur.j < jend) {
+    if (computes && cur.j < jend) {
       const char* Kl = k_ring + slot_k * T::kBytes;
       const char* Sl = s_ring + slot_s * kDsTileBytes;
+      // MFMA n: key step kc = n / kDB, feature block db = n % kDB; the K fragments are read kLead MFMAs ahead, the
+      // four dS fragments up front (order pinned, see the forward)
+      constexpr int kN = 4 * kDB, kLead = 4;
+      h8 bfrag[4], afrag[kLead];
 #pragma unroll
-      for (int c16 = 0; c16 < 4; ++c16) {
-        const h8 bfrag = s_frag(Sl, c16);
+      for (int kc = 0; kc < 4; ++kc) bfrag[kc] = s_frag(Sl, kc);
 #pragma unroll
-        for (int db = 0; db < kDBW; ++db)
-          acc[db] = mfma(swz_cols<D>(Kl, c16, dh * kDBW + db, c_off), bfrag, acc[db]);
+      for (int n = 0; n < kLead; ++n) afrag[n] = swz_cols<D>(Kl, n / kDB, n % kDB, c_off);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int n = 0; n < kN; ++n) {
+        acc[n % kDB] = mfma(afrag[n % kLead], bfrag[n / kDB], acc[n % kDB]);
+        if (n + kLead < kN) afrag[n % kLead] = swz_cols<D>(Kl, (n + kLead) / kDB, (n + kLead) % kDB, c_off);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if (cur.j == cur.nt - 1) {  // the block's last tile: its rows leave through this wave's staging tile
-      half_t* out = dQ + cur.out_off + dh * (D / 2);
+    if (computes && cur.j == cur.nt - 1) {
+      // the block's last tile: the wave's rows leave, staged where its own part of the tile was (rows 0..15 in
+      // the pieces of keys 0..31, rows 16..31 in those of keys 32..63); the slot is not refilled before the
+      // barrier of the next tile
+      char* stage = s_ring + slot_s * kDsTileBytes + own_pieces;
+      half_t* out = dQ + cur.out_off;
       const int row0 = cur.mblk * kDsBlockQ + qb * kResident;
 #pragma unroll
-      for (int part = 0; part < kDBW; ++part) {
+      for (int part = 0; part < kDB; ++part) {
         store_resident<kDsStageD>(out + part * kDsStageD, rs, row0, N, *reinterpret_cast<const f16v(*)[1]>(&acc[part]),
-                                  scale, lane, stage, my_row);
+                                  scale, lane, stage, my_row, 8192);
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[part][r] = 0.f;
       }
@@ -1906,8 +1938,13 @@ int launch_backward(int passes, bool spill, const void* q, const void* k, const 
   const float c = scale * kLog2e;
   auto dq_pass = [&]() {
     if (spill) {
-      const int nqb = np / kDsBlockQ, total = nqb * batch * head;
-      return launch(fmha_bwd_dq_spill_kernel<D, CAUSAL>, persistent_grid(total), kDsThreads, stream,
+      // two panels per block when that leaves every work group at least four blocks to balance its load with
+      const int nqb2 = (n + 2 * kDsPanelQ - 1) / (2 * kDsPanelQ), total2 = nqb2 * batch * head;
+      if (total2 >= 4 * persistent_grid(total2))
+        return launch(fmha_bwd_dq_spill_kernel<D, CAUSAL, 2>, persistent_grid(total2), ds_threads(2), stream,
+                      (const half_t*)k, ks, (const half_t*)ds, np, (half_t*)dq, head, n, nqb2, total2, scale);
+      const int nqb = np / kDsPanelQ, total = nqb * batch * head;
+      return launch(fmha_bwd_dq_spill_kernel<D, CAUSAL, 1>, persistent_grid(total), ds_threads(1), stream,
                     (const half_t*)k, ks, (const half_t*)ds, np, (half_t*)dq, head, n, nqb, total, scale);
     }
     const int nmb = (n + kDqBlockQ - 1) / kDqBlockQ;

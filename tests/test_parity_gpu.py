@@ -399,6 +399,35 @@ def test_spill_and_recompute_backward_agree(lib, B, H, N, D, causal):
     assert torch.isfinite(dq_s).all()
 
 
+TWO_PANEL_CASES = [  # B, H, N, D, causal: at least 1024 blocks of 256 queries
+    (8, 32, 1024, 128, True), (7, 32, 1100, 64, True), (4, 64, 1000, 64, False), (7, 32, 1100, 128, False),
+    (8, 32, 777, 128, True),
+]
+
+
+@pytest.mark.parametrize("B,H,N,D,causal", TWO_PANEL_CASES)
+def test_spill_backward_with_many_blocks(lib, B, H, N, D, causal):
+    """With enough blocks to go round, the dQ pass over the spilled dS takes 256 queries per block instead of 128
+    (a K tile then serves twice as many queries).  Shapes that select it, with ragged ends, an odd number of
+    128-query panels (the second half of the last block is then empty) and both maskings: dK and dV are bit-equal
+    to the minimum-workspace path, dQ equal to rounding, and batch 0 matches the oracle."""
+    scale = 1.0 / math.sqrt(D)
+    q, k, v, do = ao.make_inputs(B, N, H, D, seed=3 * N + D)
+    print(f"two-panel spill B{B} H{H} N{N} D{D} causal={causal}", flush=True)
+    assert ((N + 255) // 256) * B * H >= 1024
+    qg, kg, vg, dog = (t.cuda() for t in (q, k, v, do))
+    out, lse = abi.forward(lib, qg, kg, vg, scale, causal)
+    dq_s, dk_s, dv_s, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal)
+    dq_r, dk_r, dv_r, _ = abi.backward(lib, qg, kg, vg, out, dog, lse, scale, causal, min_workspace=True)
+    torch.cuda.synchronize()
+    assert torch.equal(dk_s, dk_r) and torch.equal(dv_s, dv_r)
+    assert (dq_s.float() - dq_r.float()).abs().max().item() <= 2e-3
+    assert torch.isfinite(dq_s).all()
+    dq_ref, dk_ref, dv_ref = ao.attention_backward(q[:1], k[:1], v[:1], do[:1], scale, causal)
+    assert _err(dq_s[:1], dq_ref) <= G_TOL
+    assert _err(dk_s[:1], dk_ref) <= G_TOL and _err(dv_s[:1], dv_ref) <= G_TOL
+
+
 def _forward_oracle_in_row_chunks(q, k, v, scale, causal, chunk=2048):
     """attention_oracle.attention_forward for ONE (batch, head) slice, evaluated in chunks of query rows so that
     the score matrix in memory is chunk x N (fp32) instead of N x N; same formulas (test.py:13-26)."""
