@@ -1938,9 +1938,9 @@ int launch_backward(int passes, bool spill, const void* q, const void* k, const 
   const float c = scale * kLog2e;
   auto dq_pass = [&]() {
     if (spill) {
-      // two panels per block when that leaves every work group at least four blocks to balance its load with
+      // two panels per block when that leaves every work group at least two blocks (a heavy and a light one)
       const int nqb2 = (n + 2 * kDsPanelQ - 1) / (2 * kDsPanelQ), total2 = nqb2 * batch * head;
-      if (total2 >= 4 * persistent_grid(total2))
+      if (total2 >= 2 * persistent_grid(total2))
         return launch(fmha_bwd_dq_spill_kernel<D, CAUSAL, 2>, persistent_grid(total2), ds_threads(2), stream,
                       (const half_t*)k, ks, (const half_t*)ds, np, (half_t*)dq, head, n, nqb2, total2, scale);
       const int nqb = np / kDsPanelQ, total = nqb * batch * head;
