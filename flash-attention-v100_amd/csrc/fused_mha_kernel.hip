@@ -294,6 +294,28 @@ __device__ __forceinline__ h8 swz_cols(const char* tile, int c16, int db, const 
   return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
+// The same reads through LDS addresses formed by the caller (tile + off[e]) and hidden from the optimiser:
+// seen whole, it may split tile + off[e] + constant into a loop-invariant part per fragment, kept in a
+// register each (and spilled), and the ring slot; opaque, the constant is the instruction's immediate offset.
+__device__ __forceinline__ unsigned opaque_lds_address(const char* p) {
+  unsigned a = (unsigned)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+  asm volatile("" : "+v"(a));
+  return a;
+}
+template <int D>
+__device__ __forceinline__ h8 swz_rows_at(unsigned a_even, unsigned a_odd, int rb, int kk) {
+  typedef __attribute__((address_space(3))) h8 lds_h8;
+  return *(const lds_h8*)(uintptr_t)(((kk & 1) ? a_odd : a_even) + (unsigned)SwzTile<D>::block_off(2 * rb, kk >> 1));
+}
+template <int D>
+__device__ __forceinline__ h8 swz_cols_at(unsigned a0, unsigned a1, int c16, int db) {
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const unsigned o = SwzTile<D>::block_off(c16, db);
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(uintptr_t)(a0 + o));
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(uintptr_t)(a1 + o));
+  return __builtin_bit_cast(h8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
 // s_waitcnt vmcnt(N) with the other counters left alone.  Issued through the
 // builtin (not inline asm) so that the compiler's wait-count bookkeeping sees it.
 template <int N>
@@ -1368,36 +1390,37 @@ fmha_bwd_dkdv_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ K,
 
   // first GEMM of a tile: rows of Q (role A) or dO (role B) against the resident
   // rows, on top of what x holds
+  // Both GEMMs read their LDS fragments kLead MFMAs ahead of their use, in an order that is written out and
+  // pinned (see the forward: scheduling hints alone are dropped when registers get scarce).
+  constexpr int kLead = 4;
   auto gemm1 = [&](const char* tile_lds, f16v (&x)[2]) __attribute__((always_inline)) {
+    const unsigned a0 = opaque_lds_address(tile_lds + r_off[0]), a1 = opaque_lds_address(tile_lds + r_off[1]);
+    constexpr int kN = 2 * G::kKSteps;  // MFMA n: row block rb = n & 1, feature step kk = n >> 1
+    h8 frag[kLead];
 #pragma unroll
-    for (int kk = 0; kk < G::kKSteps; ++kk) {
+    for (int n = 0; n < kLead; ++n) frag[n] = swz_rows_at<D>(a0, a1, n & 1, n >> 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb) x[rb] = mfma(swz_rows<D>(tile_lds, rb, kk, r_off), rf[kk], x[rb]);
+    for (int n = 0; n < kN; ++n) {
+      x[n & 1] = mfma(frag[n % kLead], rf[n >> 1], x[n & 1]);
+      if (n + kLead < kN) frag[n % kLead] = swz_rows_at<D>(a0, a1, (n + kLead) & 1, (n + kLead) >> 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    constexpr int kN = 2 * G::kKSteps, kLead = 4;
-    __builtin_amdgcn_sched_group_barrier(0x100, kLead, 0);
-#pragma unroll
-    for (int n = 0; n < kN - kLead; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
   // second GEMM: columns of dO (role A) or Q (role B) against the fp16 operand y
   auto gemm2 = [&](const char* tile_lds, const h8 (&y)[4]) __attribute__((always_inline)) {
+    const unsigned a0 = opaque_lds_address(tile_lds + c_off[0]), a1 = opaque_lds_address(tile_lds + c_off[1]);
+    constexpr int kDB = G::kDBlocks, kN = 4 * kDB;  // MFMA n: chunk c16 = n / kDB, feature block db = n % kDB
+    h8 frag[kLead];
 #pragma unroll
-    for (int c16 = 0; c16 < 4; ++c16) {
+    for (int n = 0; n < kLead; ++n) frag[n] = swz_cols_at<D>(a0, a1, n / kDB, n % kDB);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int db = 0; db < G::kDBlocks; ++db) acc[db] = mfma(swz_cols<D>(tile_lds, c16, db, c_off), y[c16], acc[db]);
+    for (int n = 0; n < kN; ++n) {
+      acc[n % kDB] = mfma(frag[n % kLead], y[n / kDB], acc[n % kDB]);
+      if (n + kLead < kN) frag[n % kLead] = swz_cols_at<D>(a0, a1, (n + kLead) / kDB, (n + kLead) % kDB);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    constexpr int kN = 4 * G::kDBlocks, kLead = 4;
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kLead, 0);
-#pragma unroll
-    for (int n = 0; n < kN - kLead; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, kLead, 0);
   };
   // P = exp2(S*c - lse2), fp16, in B-operand order.  MASKED tiles straddle the
   // diagonal or the end of the sequence.
